@@ -127,6 +127,16 @@ PROTOTYPES = {
     "exl2_window_attn": (ci, [vp, vp, vp, vp, vp, vp, vp, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, ci, ci, vp]),
     "exl2_window_attn_tiles_supported": (ci, [ci, ci]),
     "exl2_window_attn_tiles": (ci, [vp, vp, vp, vp, vp, vp, vp, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, vp, vp, vp, ci, ci, vp, vp, ci, ci, ci, ci, ci, ci, vp]),
+    # variants of the windowed attention (chunked mask, soft cap, one gate per head, query-only rows)
+    "exl2_kv_rot_append_ex": (ci, [vp, ci, ci, ci, ci, vp, vp, vp, vp, vp, vp, vp, cf, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, vp]),
+    "exl2_window_attn_ex": (ci, [vp, vp, vp, vp, vp, vp, vp, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, ci, ci, ci, cf, ci, vp]),
+    "exl2_window_attn_tiles_ex": (ci, [vp, vp, vp, vp, vp, vp, vp, ci, vp, ci, ci, vp, vp, vp, ci, ci, ci, vp, vp, vp, ci, ci, vp, vp, ci, ci, ci, ci, ci, ci, ci, cf, ci, vp]),
+    # scalar-gain RMS norm + token shift, sigmoid router (csrc/rowops.hip); decaying linear attention (csrc/wkv.hip)
+    "exl2_add_rms_shift": (ci, [vp, vp, vp, ci, cf, cf, vp, vp, vp, vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]),
+    "exl2_span_last_rows": (ci, [vp, ci, vp, ci, vp, vp, ci, vp, vp]),
+    "exl2_moe_route_sigmoid": (ci, [vp, vp, vp, ci, ci, ci, cf, vp, vp, vp, vp]),
+    "exl2_wkv_mix": (ci, [vp, vp, vp, ci, vp, cll, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]),
+    "exl2_wkv_scan": (ci, [vp, vp, vp, vp, ci, vp, ci, vp, vp, vp, ci, ci, vp, vp, vp, ci, vp, vp, ci, ci, ci, cf, vp]),
     # graphs
     "exl2_graph_begin_capture": (ci, [vp]),
     "exl2_graph_end_capture": (ci, [vp, C.POINTER(vp)]),

@@ -213,14 +213,19 @@ class SlotState:
 
 class LayerStates:
     """What a stack of unlike mixers keeps between steps: per layer whatever its mixer's `make_state(pool, dtype)` built (PagedKV for
-    attention, SlotState for recurrent mixers), all over ONE PagePool, so a request's pages and its slot are handed out and taken
+    attention, SlotState for recurrent mixers, None for a layer that reads another layer's rows), all over ONE PagePool, so a request's pages and its slot are handed out and taken
     back together."""
 
-    def __init__(self, pool: PagePool, per_layer: dict):
+    def __init__(self, pool: PagePool, per_layer: dict, norm_states: dict | None = None):
         self.pool, self.per_layer = pool, dict(per_layer)
+        self.norm_states = dict(norm_states or {})            # layer -> what the norm in front of its mixer keeps per slot (token shift)
 
     def layer(self, layer_idx: int):
         return self.per_layer[layer_idx]
 
+    def norm_state(self, layer_idx: int):
+        return self.norm_states.get(layer_idx)
+
     def footprint(self) -> int:
-        return sum(t.numel() * t.element_size() for st in self.per_layer.values() if st is not None for t in st.tensors())
+        states = list(self.per_layer.values()) + list(self.norm_states.values())
+        return sum(t.numel() * t.element_size() for st in states if st is not None for t in st.tensors())

@@ -63,9 +63,13 @@ class LayeredConfig:
     postln_alpha: float = 1.0
     embedding_scale: float = 1.0
     layers: list = field(default_factory=list)
-    residual: str = "post_rms"        # "post_rms": x <- rms_norm(alpha x + f(x)) (1 + w);  "pre_ln": x <- x + f(layer_norm(x))
+    # "post_rms": x <- rms_norm(alpha x + f(x)) (1 + w);  "pre_ln": x <- x + f(layer_norm(x));
+    # "pre_rms_shift": x <- x + f(shift(rms_norm(x) * g)), g ONE number per norm, shift = a blend with the previous token's normed row
+    residual: str = "post_rms"
     tied_head: bool = False           # logits from the embedding table itself (no `head` tensor)
     logit_softcap: float = 0.0        # > 0: logits <- c tanh(logits / c)
+    logit_scale: float = 1.0          # logits <- logits * s
+    attention_mask: str = "window"    # what an attention layer's mask.size means: "window" (sliding) or "chunk" (blocks from position 0)
 
     @staticmethod
     def from_dict_prenorm(d: dict) -> "LayeredConfig":
@@ -75,6 +79,19 @@ class LayeredConfig:
                                 norm_eps=float(d["norm"]["eps"]), embedding_scale=float(d["embedding"]["scale"]),
                                 layers=list(d["layers"]), residual="pre_ln", tied_head=True,
                                 logit_softcap=float(d.get("logit_softcap") or 0.0))
+        except KeyError as e:
+            raise RuntimeError(f"config.json: missing key {e}") from e
+        if cfg.vocab <= 0 or cfg.width <= 0 or not cfg.layers:
+            raise RuntimeError("config.json: vocab, width and layers must be given")
+        return cfg
+
+    @staticmethod
+    def from_dict_prerms_shift(d: dict) -> "LayeredConfig":
+        """pre-norm stacks with scalar-gain RMS norms and a token shift in front of every mixer, a `head` matrix and scaled logits"""
+        try:
+            cfg = LayeredConfig(architecture=str(d["architecture"]), vocab=int(d["vocab"]), width=int(d["width"]),
+                                norm_eps=float(d["norm"]["eps"]), layers=list(d["layers"]), residual="pre_rms_shift",
+                                logit_scale=float(d.get("logit_scale", 1.0)), attention_mask="chunk")
         except KeyError as e:
             raise RuntimeError(f"config.json: missing key {e}") from e
         if cfg.vocab <= 0 or cfg.width <= 0 or not cfg.layers:

@@ -12,14 +12,18 @@
 // A call may be batched over blockIdx.z (per-head projections: element offsets per batch for x, w, y, aux) or GROUPED (sparse MoE
 // at many rows: batch z = expert z multiplies the rows listed for it, counts and lists in device memory, no host round trip).
 // Epilogues fold the layer's elementwise steps into the producing linear: acc * sigmoid(aux) (output gate), silu(aux) * acc
-// (gated MLP), the clamped gated unit min(aux, L) * sigmoid(1.702 min(aux, L)) * (clamp(acc, -L, L) + 1), relu(acc)^2 and the soft
-// cap L tanh(acc / L); a bias vector (fp32, one value per output column) is added to the accumulator first.
+// (gated MLP), the clamped gated unit min(aux, L) * sigmoid(1.702 min(aux, L)) * (clamp(acc, -L, L) + 1), relu(acc)^2, the soft
+// cap L tanh(acc / L), a plain scale L acc, tanh(acc), and relu(aux[row] acc)^2 (an expert whose INPUT carries the router's weight:
+// W (s h) = s (W h)); a bias vector (fp32, one value per output column) is added to the accumulator first.
 #include "hw.h"
 #include "errors.h"
 
 enum { DENSE_BF16 = 0, DENSE_F32 = 1 };
-enum { EPI_NONE = 0, EPI_MUL_SIGMOID_AUX = 1, EPI_SILU_AUX_MUL = 2, EPI_CLAMPED_GLU = 3, EPI_RELU_SQUARED = 4, EPI_SOFT_CAP = 5 };
-#define EPI_READS_AUX(e) ((e) >= EPI_MUL_SIGMOID_AUX && (e) <= EPI_CLAMPED_GLU)
+enum { EPI_NONE = 0, EPI_MUL_SIGMOID_AUX = 1, EPI_SILU_AUX_MUL = 2, EPI_CLAMPED_GLU = 3, EPI_RELU_SQUARED = 4, EPI_SOFT_CAP = 5,
+       EPI_SCALE = 6, EPI_TANH = 7, EPI_ROW_SCALED_RELU_SQUARED = 8, EPI_LAST = 8 };
+#define EPI_ROW_AUX(e) ((e) == EPI_ROW_SCALED_RELU_SQUARED)          // aux holds ONE value per row (ldaux apart), not one per output
+#define EPI_READS_AUX(e) (((e) >= EPI_MUL_SIGMOID_AUX && (e) <= EPI_CLAMPED_GLU) || EPI_ROW_AUX(e))
+#define EPI_AUX_COL(e, n) (EPI_ROW_AUX(e) ? 0 : (n))
 
 struct LinArgs
 {
@@ -78,6 +82,9 @@ DEV float lin_epilogue(int epi, float acc, float aux, float limit)
     }
     if (epi == EPI_RELU_SQUARED) { const float r = fmaxf(acc, 0.0f); return r * r; }
     if (epi == EPI_SOFT_CAP) return limit * tanhf(acc / limit);
+    if (epi == EPI_SCALE) return acc * limit;
+    if (epi == EPI_TANH) return tanhf(acc);
+    if (epi == EPI_ROW_SCALED_RELU_SQUARED) { const float r = fmaxf(acc * aux, 0.0f); return r * r; }
     return acc;
 }
 
@@ -145,7 +152,7 @@ KERNEL void __launch_bounds__(256) lin_rows_kernel(const LinArgs a)
             const int r = r0 + m;
             if (r >= a.M) break;
             float aux = 0.0f;
-            if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + (long long)r * a.ldaux + n];
+            if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + (long long)r * a.ldaux + EPI_AUX_COL(a.epi, n)];
             st1<TY>((TY*)a.y + (long long)z * a.syb + (long long)r * a.ldy + n, lin_epilogue(a.epi, acc[m] + (a.bias ? a.bias[n] : 0.0f), aux, a.limit));
         }
     }
@@ -214,7 +221,7 @@ KERNEL void __launch_bounds__(256) lin_tile_kernel(const LinArgs a)
             const int n = n0 + tx * 4 + j;
             if (n >= a.N) continue;
             float aux = 0.0f;
-            if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + r * a.ldaux + n];
+            if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + r * a.ldaux + EPI_AUX_COL(a.epi, n)];
             st1<TY>((TY*)a.y + (long long)z * a.syb + r * a.ldy + n, lin_epilogue(a.epi, acc[i][j] + (a.bias ? a.bias[n] : 0.0f), aux, a.limit));
         }
     }
@@ -284,7 +291,7 @@ KERNEL void __launch_bounds__(256) lin_mfma_kernel(const LinArgs a)
                 const int n = n0 + 16 * j + li;
                 if (n >= a.N) continue;
                 float aux = 0.0f;
-                if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + row * a.ldaux + n];
+                if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + row * a.ldaux + EPI_AUX_COL(a.epi, n)];
                 st1<TY>((TY*)a.y + (long long)z * a.syb + row * a.ldy + n, lin_epilogue(a.epi, acc[i][j][r] + (a.bias ? a.bias[n] : 0.0f), aux, a.limit));
             }
         }
@@ -381,7 +388,7 @@ KERNEL void __launch_bounds__(256) lin_mfma_tile_kernel(const LinArgs a)
                 const int n = n0 + wn + 16 * j + li;
                 if (n >= a.N) continue;
                 float aux = 0.0f;
-                if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + row * a.ldaux + n];
+                if (EPI_READS_AUX(a.epi)) aux = a.aux[(long long)z * a.sauxb + row * a.ldaux + EPI_AUX_COL(a.epi, n)];
                 st1<TY>((TY*)a.y + (long long)z * a.syb + row * a.ldy + n, lin_epilogue(a.epi, acc[i][j][r] + (a.bias ? a.bias[n] : 0.0f), aux, a.limit));
             }
         }
@@ -446,7 +453,7 @@ extern "C" int exl2_dense_linear_bias(const void* x, const void* w, const float*
     EXL2_REQUIRE(dtype == DENSE_BF16 || dtype == DENSE_F32, "dense_linear: dtype must be 0 (bfloat16) or 1 (float32)");
     EXL2_REQUIRE(M >= 0 && N > 0 && K > 0 && batch > 0 && x_div > 0, "dense_linear: bad shape %d x %d x %d, batch %d", M, N, K, batch);
     EXL2_REQUIRE(ldx >= K || x_div > 0, "dense_linear: ldx"); EXL2_REQUIRE(ldw >= K && ldy > 0, "dense_linear: leading dimensions");
-    EXL2_REQUIRE(epi >= EPI_NONE && epi <= EPI_SOFT_CAP, "dense_linear: unknown epilogue %d", epi);
+    EXL2_REQUIRE(epi >= EPI_NONE && epi <= EPI_LAST, "dense_linear: unknown epilogue %d", epi);
     EXL2_REQUIRE(!EPI_READS_AUX(epi) || aux, "dense_linear: the epilogue needs aux");
     EXL2_REQUIRE(epi != EPI_SOFT_CAP || limit > 0.0f, "dense_linear: the soft cap needs a positive limit");
     EXL2_REQUIRE(!bias || (batch == 1 && !w_sel && !grp_count), "dense_linear: a bias goes with a plain (one-slab) call");

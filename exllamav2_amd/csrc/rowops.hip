@@ -4,8 +4,10 @@
 //   * the pre-norm residual step  x <- x + y  with the layer norm (weight and bias) that feeds the next sublayer,
 //   * the post-norm residual step  x <- norm(alpha x + y) (1 + w), where y is a linear's fp32 output or the weighted sum of a
 //     token's chosen experts (identity experts contribute the token's own x),
-//   * the sparse-MoE router (softmax over all experts, selection by score + correction, weights from the uncorrected scores) and
-//     the per-expert row lists the grouped linear reads.
+//   * the pre-norm residual step  x <- x + y (+ the sum of a token's expert outputs)  with an RMS norm whose gain is ONE number and
+//     a token shift  h + (h' - h) * shift  towards the previous token's normed row (kept per sequence slot),
+//   * the sparse-MoE router (softmax over all experts, selection by score + correction, weights from the uncorrected scores; or
+//     sigmoid scores, selection and weights by the scores themselves) and the per-expert row lists the grouped linear reads.
 // Element type T of weights / operand copies: u16 = bfloat16 bits, float.
 #include "hw.h"
 #include "errors.h"
@@ -226,14 +228,104 @@ KERNEL void __launch_bounds__(256) add_layer_norm_vec_kernel(const LayerNormArgs
     }
 }
 
+// ---- x <- x + y, RMS norm with a scalar gain, token shift --------------------------------------------------------------------------
+// hn[r] = x[r] / sqrt(mean(x[r]^2) + eps) * gain after the stream took the sublayer's output: y (nullable) and / or the sum of the
+// `top` expert outputs of the row (moe_y rows r * top .. + top, nullable).  With a shift vector the consumer reads
+// out[r] = hn[r] + (hn' - hn[r]) * shift, hn' = the normed row of the sequence's previous token: the row in front of r when that
+// belongs to the same sequence, else what the slot keeps (prev fp32 [slots, width]), zeros at position 0.  Steps whose spans are
+// single rows (decoding) do everything in ONE launch and roll the slot; otherwise hn goes to a buffer, a second launch shifts
+// (every row independent) and a third rolls the slots from the spans' last rows -- nothing reads a slot after it was rolled.
+
+struct RmsShiftArgs
+{
+    float* x; const float* y; const float* moe_y; int top;
+    float* hn;                               // fp32 [rows, width] (multi-row spans with a shift), else unused
+    void* out; int out_f32;                  // [rows, width] operand dtype or fp32
+    const void* shift;                       // [width] operand dtype (nullable: out = hn)
+    float* prev;                             // fp32 [slots, width]
+    const int* row_seq; const int* row_pos; const int* row_idx;
+    int width; float gain, eps; int fused;   // fused: single-row spans, shift and slot roll inside the norm launch
+};
+
+template <typename T>
+KERNEL void __launch_bounds__(256) add_rms_shift_kernel(const RmsShiftArgs a)
+{
+    DYN_SMEM(smem);
+    SHARED float part[4];
+    float* v = (float*)smem;
+    const int r = bid_x();
+    const long long src = a.row_idx ? a.row_idx[r] : r;
+    float* xr = a.x + src * a.width;
+    float ss = 0.0f;
+    for (int i = tid(); i < a.width; i += 256)
+    {
+        float xv = xr[i];
+        if (a.y || a.moe_y)
+        {
+            if (a.y) xv += a.y[src * a.width + i];
+            for (int k = 0; k < (a.moe_y ? a.top : 0); k++) xv += a.moe_y[(src * a.top + k) * a.width + i];
+            xr[i] = xv;
+        }
+        v[i] = xv;
+        ss = fmaf(xv, xv, ss);
+    }
+    if (!a.out && !a.hn) return;                                 // only the addition
+    ss = block_sum_256(ss, part);
+    const float mul = a.gain / sqrtf(ss / (float)a.width + a.eps);
+    if (a.shift && !a.fused)
+    {
+        for (int i = tid(); i < a.width; i += 256) a.hn[(long long)r * a.width + i] = v[i] * mul;
+        return;
+    }
+    float* pv = nullptr; bool first = true;
+    if (a.shift) { pv = a.prev + (long long)a.row_seq[r] * a.width; first = a.row_pos[r] == 0; }
+    for (int i = tid(); i < a.width; i += 256)
+    {
+        const float hn = v[i] * mul;
+        float o = hn;
+        if (a.shift)
+        {
+            const float hp = first ? 0.0f : pv[i];
+            o = fmaf(hp - hn, ro_ld<T>((const T*)a.shift + i), hn);
+            pv[i] = hn;
+        }
+        if (a.out_f32) ((float*)a.out)[(long long)r * a.width + i] = o; else ro_st<T>((T*)a.out + (long long)r * a.width + i, o);
+    }
+}
+
+// grid (rows, width / 256): out[r] = hn[r] + (hn' - hn[r]) * shift
+template <typename T>
+KERNEL void __launch_bounds__(256) token_shift_kernel(const RmsShiftArgs a)
+{
+    const int r = bid_x(), i = bid_y() * 256 + tid();
+    if (i >= a.width) return;
+    const int pos = a.row_pos[r], sq = a.row_seq[r];
+    float hp = 0.0f;
+    if (pos > 0) hp = (r > 0 && a.row_seq[r - 1] == sq) ? a.hn[(long long)(r - 1) * a.width + i] : a.prev[(long long)sq * a.width + i];
+    const float hn = a.hn[(long long)r * a.width + i];
+    const float o = fmaf(hp - hn, ro_ld<T>((const T*)a.shift + i), hn);
+    if (a.out_f32) ((float*)a.out)[(long long)r * a.width + i] = o; else ro_st<T>((T*)a.out + (long long)r * a.width + i, o);
+}
+
+// grid (spans, width / 256): slot of span s <- row (last of the span) of src fp32 [rows, ld]
+KERNEL void __launch_bounds__(256) span_last_row_kernel(const float* src, int ld, float* slot_rows, int width, const int* span_row0,
+                                                         const int* span_rows, const int* row_seq)
+{
+    const int s = bid_x(), i = bid_y() * 256 + tid();
+    if (i >= width) return;
+    const int last = span_row0[s] + span_rows[s] - 1;
+    slot_rows[(long long)row_seq[last] * width + i] = src[(long long)last * ld + i];
+}
+
 // ---- router -----------------------------------------------------------------------------------------------------------------
 // One wave per token.  logits fp32 [rows, n_total]; scores = softmax over all n_total; the `top` largest (score + correction) win
-// (first index on a tie); weight = score / (sum of the chosen scores + 1e-20) * scale.
+// (first index on a tie); weight = score / (sum of the chosen scores + 1e-20) * scale.  sigmoid_scores: scores = sigmoid(logits),
+// each on its own, and the weights are the chosen scores times scale (no renormalisation).
 
 #define ROUTE_MAX_PER_LANE 8
 
 KERNEL void __launch_bounds__(64) moe_route_kernel(const float* logits, const float* correction, int* ids, float* wts,
-                                                    int n_total, int top, float scale)
+                                                    int n_total, int top, float scale, int sigmoid_scores)
 {
     const int r = bid_x();
     const int lane = lane_id();
@@ -252,10 +344,11 @@ KERNEL void __launch_bounds__(64) moe_route_kernel(const float* logits, const fl
     for (int i = 0; i < ROUTE_MAX_PER_LANE; i++)
     {
         const int e = lane + 64 * i;
-        s[i] = e < n_total ? expf(s[i] - mx) : 0.0f;
+        if (sigmoid_scores) s[i] = e < n_total ? 1.0f / (1.0f + expf(-s[i])) : 0.0f;
+        else s[i] = e < n_total ? expf(s[i] - mx) : 0.0f;
         sum += s[i];
     }
-    sum = wave_allreduce_add(sum);
+    sum = sigmoid_scores ? 1.0f : wave_allreduce_add(sum);
     #pragma unroll
     for (int i = 0; i < ROUTE_MAX_PER_LANE; i++)
     {
@@ -290,7 +383,7 @@ KERNEL void __launch_bounds__(64) moe_route_kernel(const float* logits, const fl
     if (lane < top)
     {
         ids[r * top + lane] = my_id;
-        wts[r * top + lane] = my_w / (chosen_sum + 1e-20f) * scale;
+        wts[r * top + lane] = sigmoid_scores ? my_w * scale : my_w / (chosen_sum + 1e-20f) * scale;
     }
 }
 
@@ -420,15 +513,30 @@ extern "C" int exl2_add_layer_norm(float* x, const float* y, const void* w, cons
     return EXL2_OK;
 }
 
+static int moe_route_any(const float* logits, const float* correction, int* ids, float* wts, int rows, int n_total, int top,
+                         float scale, int n_real, int* grp_count, int* grp_offset, int* grp_rows, int sigmoid_scores, void* stream);
+
 extern "C" int exl2_moe_route_scored(const float* logits, const float* correction, int* ids, float* wts, int rows, int n_total, int top,
                                      float scale, int n_real, int* grp_count, int* grp_offset, int* grp_rows, void* stream)
+{
+    return moe_route_any(logits, correction, ids, wts, rows, n_total, top, scale, n_real, grp_count, grp_offset, grp_rows, 0, stream);
+}
+
+extern "C" int exl2_moe_route_sigmoid(const float* logits, int* ids, float* wts, int rows, int n_total, int top, float scale,
+                                      int* grp_count, int* grp_offset, int* grp_rows, void* stream)
+{
+    return moe_route_any(logits, nullptr, ids, wts, rows, n_total, top, scale, n_total, grp_count, grp_offset, grp_rows, 1, stream);
+}
+
+static int moe_route_any(const float* logits, const float* correction, int* ids, float* wts, int rows, int n_total, int top,
+                         float scale, int n_real, int* grp_count, int* grp_offset, int* grp_rows, int sigmoid_scores, void* stream)
 {
     EXL2_REQUIRE(logits && ids && wts, "moe_route_scored: null operand");
     EXL2_REQUIRE(n_total > 0 && n_total <= 64 * ROUTE_MAX_PER_LANE, "moe_route_scored: %d experts (at most %d)", n_total, 64 * ROUTE_MAX_PER_LANE);
     EXL2_REQUIRE(top > 0 && top <= 64 && top <= n_total, "moe_route_scored: top %d of %d", top, n_total);
     EXL2_REQUIRE(n_real >= 0 && n_real <= n_total, "moe_route_scored: %d experts with weights of %d", n_real, n_total);
     if (rows <= 0) return EXL2_OK;
-    LAUNCH(moe_route_kernel, dim3(rows), dim3(64), 0, stream, logits, correction, ids, wts, n_total, top, scale);
+    LAUNCH(moe_route_kernel, dim3(rows), dim3(64), 0, stream, logits, correction, ids, wts, n_total, top, scale, sigmoid_scores);
     if (grp_count)
     {
         EXL2_REQUIRE(grp_offset && grp_rows, "moe_route_scored: grouped lists need offsets and rows");
@@ -438,6 +546,59 @@ extern "C" int exl2_moe_route_scored(const float* logits, const float* correctio
             LAUNCH(moe_fill_kernel, dim3(n_real), dim3(64), 0, stream, (const int*)ids, rows * top, (const int*)grp_count, grp_offset, grp_rows);
         }
     }
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+extern "C" int exl2_add_rms_shift(float* x, const float* y, const float* moe_y, int top, float gain, float eps, const void* shift,
+                                  float* prev, float* hn, void* out, int out_f32, const int* row_seq, const int* row_pos,
+                                  const int* row_idx, const int* span_row0, const int* span_rows, int spans, int max_span_rows,
+                                  int dtype, int rows, int width, void* stream)
+{
+    EXL2_REQUIRE(x, "add_rms_shift: null stream");
+    EXL2_REQUIRE(dtype == 0 || dtype == 1, "add_rms_shift: dtype must be 0 (bfloat16) or 1 (float32)");
+    EXL2_REQUIRE(!moe_y || top > 0, "add_rms_shift: expert outputs need their count per row");
+    EXL2_REQUIRE(out || y || moe_y, "add_rms_shift: neither an addition nor a norm");
+    EXL2_REQUIRE(!(row_idx && (y || moe_y || shift)), "add_rms_shift: gathered rows take no addition and no shift");
+    EXL2_REQUIRE(!shift || (out && prev && row_seq && row_pos && span_row0 && span_rows && spans > 0 && max_span_rows > 0),
+                 "add_rms_shift: a shift needs an output, the slots' rows and the step's spans");
+    EXL2_REQUIRE(!shift || max_span_rows == 1 || hn, "add_rms_shift: spans of several rows need the buffer of normed rows");
+    EXL2_REQUIRE(width > 0 && (size_t)width * 4 <= 160 * 1024 - 64, "add_rms_shift: row of %d values does not fit the LDS", width);
+    if (rows <= 0) return EXL2_OK;
+    RmsShiftArgs a;
+    a.x = x; a.y = y; a.moe_y = moe_y; a.top = top; a.hn = shift && max_span_rows > 1 ? hn : nullptr; a.out = out;
+    a.out_f32 = out_f32 || dtype == 1; a.shift = shift; a.prev = prev; a.row_seq = row_seq; a.row_pos = row_pos; a.row_idx = row_idx;
+    a.width = width; a.gain = gain; a.eps = eps; a.fused = shift && max_span_rows == 1;
+    const size_t smem = (size_t)width * 4;
+    if (smem > 48 * 1024)
+    {
+        static bool attr_done[EXL2_MAX_DEVICES];
+        if (exl2_first_on_device(attr_done))
+        {
+            (void)hipFuncSetAttribute((const void*)add_rms_shift_kernel<u16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)add_rms_shift_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        }
+    }
+    if (dtype == 0) LAUNCH(add_rms_shift_kernel<u16>, dim3(rows), dim3(256), smem, stream, a);
+    else LAUNCH(add_rms_shift_kernel<float>, dim3(rows), dim3(256), smem, stream, a);
+    if (shift && !a.fused)
+    {
+        const dim3 grid(rows, (width + 255) / 256);
+        if (dtype == 0) LAUNCH(token_shift_kernel<u16>, grid, dim3(256), 0, stream, a);
+        else LAUNCH(token_shift_kernel<float>, grid, dim3(256), 0, stream, a);
+        LAUNCH(span_last_row_kernel, dim3(spans, (width + 255) / 256), dim3(256), 0, stream, (const float*)hn, width, prev, width, span_row0,
+               span_rows, row_seq);
+    }
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+extern "C" int exl2_span_last_rows(const float* src, int ld, float* slot_rows, int width, const int* span_row0, const int* span_rows,
+                                   int spans, const int* row_seq, void* stream)
+{
+    EXL2_REQUIRE(src && slot_rows && span_row0 && span_rows && row_seq && width > 0 && ld >= width, "span_last_rows: bad operand");
+    if (spans <= 0) return EXL2_OK;
+    LAUNCH(span_last_row_kernel, dim3(spans, (width + 255) / 256), dim3(256), 0, stream, src, ld, slot_rows, width, span_row0, span_rows, row_seq);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;
 }

@@ -15,6 +15,10 @@
 // Rows of a step are a flat list (row r = position row_pos[r] of sequence row_seq[r]); a row's result depends only on its own
 // (sequence, position).  Scores, softmax, sums, angles and rotations are fp32.
 // Rotary layouts: halves (value i pairs with i + n / 2) or interleaved (2i with 2i + 1); angle p * freq[i], cos and sin times `amp`.
+// Variants a design may ask for (the *_ex entry points): a CHUNKED mask instead of the window -- p sees j <= p with
+// floor(j / chunk) == floor(p / chunk), chunks counted from the sequence's start --, a soft cap  c tanh(s / c)  on the scores, ONE gate
+// value per head instead of one per output value, and rows that bring queries only (a layer that attends over another layer's
+// cached keys and values).
 #include "hw.h"
 #include "errors.h"
 #include <stdint.h>
@@ -78,7 +82,8 @@ KERNEL void __launch_bounds__(256) rot_append_kernel(const RotAppendArgs a)
     const int half = a.rot_dims / 2;
     // queries and keys: (H + G) heads of `dim` values; pairs first, then the values past rot_dims
     const int per = half + (a.dim - a.rot_dims);
-    for (int i = t; i < (a.H + a.G) * per; i += 256)
+    const int kv_heads = a.k_cache ? a.G : 0;                    // no cache: the rows bring queries only
+    for (int i = t; i < (a.H + kv_heads) * per; i += 256)
     {
         const int hd = i / per, e = i % per;
         const bool is_q = hd < a.H;
@@ -102,6 +107,7 @@ KERNEL void __launch_bounds__(256) rot_append_kernel(const RotAppendArgs a)
         }
     }
     const int vhalf = a.vdim / 2;
+    if (!a.k_cache) return;
     for (int i = t; i < a.G * vhalf; i += 256)
     {
         const int g = i / vhalf, e = i % vhalf;
@@ -226,7 +232,14 @@ struct WinAttnArgs
     void* out;                               // [rows, H, vdim]
     int H, G, dim, vdim, window;
     int page_shift, pool_shift;              // log2 of page / pool where they are powers of two, else -1 (tile kernels: no divisions)
+    int chunk;                               // > 0: chunked mask (the window is not used, no pooled blocks)
+    float softcap;                           // > 0: score <- softcap * tanh(score / softcap)
+    int gate_head;                           // gate holds one value per head (at h) instead of one per output value (at h * vdim + e)
 };
+
+// first token position `pos` sees (window form: may be negative)
+DEV int wa_first_key(int pos, int window, int chunk) { return chunk > 0 ? pos - pos % chunk : pos - window + 1; }
+DEV float wa_soft_cap(float s, float cap) { return cap > 0.0f ? cap * tanhf(s / cap) : s; }
 
 DEV int wa_div(int x, int d, int shift) { return shift >= 0 ? x >> shift : x / d; }
 DEV int wa_mod(int x, int d, int shift) { return shift >= 0 ? x & (d - 1) : x % d; }
@@ -260,7 +273,7 @@ KERNEL void __launch_bounds__(256) window_attn_kernel(const WinAttnArgs a)
     for (int i = t; i < a.dim; i += 256) qv[i] = wa_ld<T>(qr + i);
     block_sync();
     const int nb = wa_blocks_seen(pos, a.window, a.pool);
-    const int j_lo = max(0, pos - a.window + 1);
+    const int j_lo = max(0, wa_first_key(pos, a.window, a.chunk));
     const int nkeys = nb + (pos - j_lo + 1);
     float m_run = a.sink ? a.sink[h] : -INFINITY, l_run = a.sink ? 1.0f : 0.0f;
     float acc[WA_MAX_V_PER_THREAD];
@@ -290,7 +303,7 @@ KERNEL void __launch_bounds__(256) window_attn_kernel(const WinAttnArgs a)
             }
             float d = 0.0f;
             for (int i = 0; i < a.dim; i++) d = fmaf(qv[i], wa_ld<T>(kr + i), d);
-            s = d;
+            s = wa_soft_cap(d, a.softcap);
         }
         const float m_new = fmaxf(m_run, wa_block_max(s, part));
         const float p = t < nc ? expf(s - m_new) : 0.0f;
@@ -322,7 +335,8 @@ KERNEL void __launch_bounds__(256) window_attn_kernel(const WinAttnArgs a)
     }
     block_sync();
     T* out = (T*)a.out + ((long long)r * a.H + h) * a.vdim;
-    const float* gt = a.gate ? a.gate + (long long)r * a.ldg + h * a.vdim : nullptr;
+    const float* gt = a.gate && !a.gate_head ? a.gate + (long long)r * a.ldg + h * a.vdim : nullptr;
+    const float hg = a.gate && a.gate_head ? 1.0f / (1.0f + expf(-a.gate[(long long)r * a.ldg + h])) : 1.0f;
     const float fpos = (float)pos;
     const int vhalf = a.vdim / 2;
     for (int i = t; i < vhalf; i += 256)
@@ -338,14 +352,14 @@ KERNEL void __launch_bounds__(256) window_attn_kernel(const WinAttnArgs a)
             u = u2; v = v2;
         }
         if (gt) { u *= 1.0f / (1.0f + expf(-gt[ia])); v *= 1.0f / (1.0f + expf(-gt[ib])); }
-        wa_st<T>(out + ia, u);
-        wa_st<T>(out + ib, v);
+        wa_st<T>(out + ia, u * hg);
+        wa_st<T>(out + ib, v * hg);
     }
     if ((a.vdim & 1) && t == 0)
     {
         float u = ov[a.vdim - 1];
         if (gt) u *= 1.0f / (1.0f + expf(-gt[a.vdim - 1]));
-        wa_st<T>(out + a.vdim - 1, u);
+        wa_st<T>(out + a.vdim - 1, u * hg);
     }
 }
 
@@ -395,7 +409,7 @@ KERNEL void __launch_bounds__(256, 2) window_attn_mfma_kernel(const WinMfmaArgs 
     const int p0 = a.row_pos[r0], p_last = p0 + n_rows - 1;
     const int* bt = a.block_table + (long long)a.row_seq[r0] * a.bt_stride;
     const int NB = wa_blocks_seen(p_last, a.window, a.pool);
-    const int j_lo = max(0, p0 - a.window + 1);
+    const int j_lo = max(0, wa_first_key(p0, a.window, a.chunk));
     const int total = NB + (p_last - j_lo + 1);
     const int n_tiles = (total + WM_BK - 1) / WM_BK;
     const u16* kc = (const u16*)a.k_cache; const u16* vc = (const u16*)a.v_cache;
@@ -428,12 +442,12 @@ KERNEL void __launch_bounds__(256, 2) window_attn_mfma_kernel(const WinMfmaArgs 
         #pragma unroll
         for (int kk = 0; kk < KK; kk++) qb[n][kk] = *(const u32x4*)(qp + 32 * kk);
         my_nb[n] = wa_blocks_seen(qpos[n], a.window, a.pool);
-        my_lo[n] = qpos[n] - a.window + 1;                      // first token this query sees (may be negative)
+        my_lo[n] = wa_first_key(qpos[n], a.window, a.chunk);    // first token this query sees (may be negative)
     }
     const bool wave_live = wv * RPW * 16 < n_rows;
     // what the wave as a whole can see: blocks below wave_nb, tokens wave_lo .. wave_hi
     const int wp0 = p0 + min(wv * RPW * 16, n_rows - 1), wp1 = p0 + min(wv * RPW * 16 + RPW * 16 - 1, n_rows - 1);
-    const int wave_nb = wa_blocks_seen(wp1, a.window, a.pool), wave_lo = wp0 - a.window + 1, wave_hi = wp1;
+    const int wave_nb = wa_blocks_seen(wp1, a.window, a.pool), wave_lo = wa_first_key(wp0, a.window, a.chunk), wave_hi = wp1;
 
     f32x4 ot[RPW][DB];
     float m_run[RPW], l_run[RPW];
@@ -547,7 +561,7 @@ KERNEL void __launch_bounds__(256, 2) window_attn_mfma_kernel(const WinMfmaArgs 
                     const int e = k0 + 16 * blk + 4 * g + r;
                     const int j = j_lo + (e - NB);
                     const bool valid = e < total && (e < NB ? e < my_nb[n] : (j <= qpos[n] && j >= my_lo[n]));
-                    const float v = valid ? st[n][blk][r] : WM_NEG_BIG;
+                    const float v = valid ? wa_soft_cap(st[n][blk][r], a.softcap) : WM_NEG_BIG;
                     sc[blk * 4 + r] = v;
                     m_loc = fmaxf(m_loc, v);
                 }
@@ -628,11 +642,12 @@ KERNEL void __launch_bounds__(256, 2) window_attn_mfma_kernel(const WinMfmaArgs 
             }
         }
         u16* op = (u16*)a.out + ((long long)qrow[n] * a.H + h) * VDIM + 4 * g;
-        const float* gt = a.gate ? a.gate + (long long)qrow[n] * a.ldg + h * VDIM + 4 * g : nullptr;
+        const float* gt = a.gate && !a.gate_head ? a.gate + (long long)qrow[n] * a.ldg + h * VDIM + 4 * g : nullptr;
+        const float hg = a.gate && a.gate_head ? 1.0f / (1.0f + expf(-a.gate[(long long)qrow[n] * a.ldg + h])) : 1.0f;
         #pragma unroll
         for (int d = 0; d < DB; d++)
         {
-            f32x4 y = ot[n][d];
+            f32x4 y = ot[n][d] * hg;
             if (gt)
             {
                 const f32x4 gv = *(const f32x4*)(gt + 16 * d);
@@ -687,7 +702,7 @@ KERNEL void __launch_bounds__(256) window_attn_decode_kernel(const WinMfmaArgs m
     const int pos = a.row_pos[r];
     const int* bt = a.block_table + (long long)a.row_seq[r] * a.bt_stride;
     const int NB = wa_blocks_seen(pos, a.window, a.pool);
-    const int j_lo = max(0, pos - a.window + 1);
+    const int j_lo = max(0, wa_first_key(pos, a.window, a.chunk));
     const int total = NB + (pos - j_lo + 1);
     const int all_steps = (total + WD_BK - 1) / WD_BK;
     const int per_split = (all_steps + m.nsplit - 1) / m.nsplit;
@@ -795,7 +810,7 @@ KERNEL void __launch_bounds__(256) window_attn_decode_kernel(const WinMfmaArgs m
             #pragma unroll
             for (int rr = 0; rr < 4; rr++)
             {
-                const float v = k0 + 16 * blk + 4 * g + rr < total ? st[blk][rr] : WM_NEG_BIG;
+                const float v = k0 + 16 * blk + 4 * g + rr < total ? wa_soft_cap(st[blk][rr], a.softcap) : WM_NEG_BIG;
                 sc[blk * 4 + rr] = v;
                 m_loc = fmaxf(m_loc, v);
             }
@@ -877,7 +892,12 @@ KERNEL void __launch_bounds__(256) window_attn_decode_kernel(const WinMfmaArgs m
             const float u2 = u * c + v * sn, v2 = v * c - u * sn;
             u = u2; v = v2;
         }
-        if (a.gate)
+        if (a.gate && a.gate_head)
+        {
+            const float hg = 1.0f / (1.0f + expf(-a.gate[(long long)r * a.ldg + hd]));
+            u *= hg; v *= hg;
+        }
+        else if (a.gate)
         {
             const float* gt = a.gate + (long long)r * a.ldg + hd * VDIM;
             u *= 1.0f / (1.0f + expf(-gt[ia])); v *= 1.0f / (1.0f + expf(-gt[ib]));
@@ -903,7 +923,8 @@ KERNEL void __launch_bounds__(64) window_attn_merge_kernel(const WinMfmaArgs m)
     }
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
     const float fpos = (float)a.row_pos[r];
-    const float* gt = a.gate ? a.gate + (long long)r * a.ldg + hd * a.vdim : nullptr;
+    const float* gt = a.gate && !a.gate_head ? a.gate + (long long)r * a.ldg + hd * a.vdim : nullptr;
+    const float hg = a.gate && a.gate_head ? 1.0f / (1.0f + expf(-a.gate[(long long)r * a.ldg + hd])) : 1.0f;
     u16* op = (u16*)a.out + ((long long)r * a.H + hd) * a.vdim;
     for (int pr = tid(); pr < a.vdim / 2; pr += 64)
     {
@@ -927,7 +948,7 @@ KERNEL void __launch_bounds__(64) window_attn_merge_kernel(const WinMfmaArgs m)
             u = u2; v = v2;
         }
         if (gt) { u *= 1.0f / (1.0f + expf(-gt[ia])); v *= 1.0f / (1.0f + expf(-gt[ib])); }
-        op[ia] = f32_to_bf16(u); op[ib] = f32_to_bf16(v);
+        op[ia] = f32_to_bf16(u * hg); op[ib] = f32_to_bf16(v * hg);
     }
 }
 
@@ -947,13 +968,44 @@ static void wd_launch(const WinMfmaArgs& m, int tiles, hipStream_t s)
 
 // ---- C ABI ----------------------------------------------------------------------------------------------------------------------
 
+extern "C" int exl2_kv_rot_append_ex(const float* f, int ld, int q_off, int k_off, int v_off, void* q_out, const float* q_scale,
+                                     void* k_cache, void* v_cache, void* k_pool, void* v_pool, const float* freq, float amp, int rot_dims,
+                                     const float* vfreq, int v_rot, int interleaved, const int* row_seq, const int* row_pos,
+                                     const int* block_table, int bt_stride, int page, int pool, int dtype, int rows, int heads,
+                                     int kv_heads, int dim, int vdim, void* stream);
+extern "C" int exl2_window_attn_ex(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
+                                   const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
+                                   const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
+                                   void* out, int dtype, int rows, int heads, int kv_heads, int dim, int vdim, int window, int chunk,
+                                   float softcap, int gate_head, void* stream);
+extern "C" int exl2_window_attn_tiles_ex(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
+                                         const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
+                                         const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
+                                         void* out, const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, float* part_o,
+                                         float* part_ml, int nsplit, int heads, int kv_heads, int dim, int vdim, int window, int chunk,
+                                         float softcap, int gate_head, void* stream);
+
 extern "C" int exl2_kv_rot_append(const float* f, int ld, int q_off, int k_off, int v_off, void* q_out, const float* q_scale,
                                   void* k_cache, void* v_cache, void* k_pool, void* v_pool, const float* freq, float amp, int rot_dims,
                                   const float* vfreq, int v_rot, int interleaved, const int* row_seq, const int* row_pos,
                                   const int* block_table, int bt_stride, int page, int pool, int dtype, int rows, int heads,
                                   int kv_heads, int dim, int vdim, void* stream)
 {
-    EXL2_REQUIRE(f && q_out && q_scale && k_cache && v_cache && freq && row_seq && row_pos && block_table, "kv_rot_append: null operand");
+    EXL2_REQUIRE(k_cache && v_cache, "kv_rot_append: null operand");
+    return exl2_kv_rot_append_ex(f, ld, q_off, k_off, v_off, q_out, q_scale, k_cache, v_cache, k_pool, v_pool, freq, amp, rot_dims, vfreq,
+                                 v_rot, interleaved, row_seq, row_pos, block_table, bt_stride, page, pool, dtype, rows, heads, kv_heads,
+                                 dim, vdim, stream);
+}
+
+extern "C" int exl2_kv_rot_append_ex(const float* f, int ld, int q_off, int k_off, int v_off, void* q_out, const float* q_scale,
+                                     void* k_cache, void* v_cache, void* k_pool, void* v_pool, const float* freq, float amp, int rot_dims,
+                                     const float* vfreq, int v_rot, int interleaved, const int* row_seq, const int* row_pos,
+                                     const int* block_table, int bt_stride, int page, int pool, int dtype, int rows, int heads,
+                                     int kv_heads, int dim, int vdim, void* stream)
+{
+    EXL2_REQUIRE(f && q_out && q_scale && freq && row_seq && row_pos && block_table, "kv_rot_append: null operand");
+    EXL2_REQUIRE((k_cache == nullptr) == (v_cache == nullptr), "kv_rot_append: keys and values go to the cache together");
+    EXL2_REQUIRE(k_cache || pool == 0, "kv_rot_append: rows that bring queries only write no pooled blocks");
     EXL2_REQUIRE(dtype == 0 || dtype == 1, "kv_rot_append: dtype must be 0 (bfloat16) or 1 (float32)");
     EXL2_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0, "kv_rot_append: bad head shape");
     EXL2_REQUIRE(rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0, "kv_rot_append: %d rotated of %d values", rot_dims, dim);
@@ -988,6 +1040,18 @@ extern "C" int exl2_window_attn(const void* q, const void* k_cache, const void* 
                                 const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
                                 void* out, int dtype, int rows, int heads, int kv_heads, int dim, int vdim, int window, void* stream)
 {
+    return exl2_window_attn_ex(q, k_cache, v_cache, k_pool, v_pool, sink, gate, ldg, vfreq, v_rot, interleaved, row_seq, row_pos,
+                               block_table, bt_stride, page, pool, out, dtype, rows, heads, kv_heads, dim, vdim, window, 0, 0.0f, 0, stream);
+}
+
+extern "C" int exl2_window_attn_ex(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
+                                   const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
+                                   const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
+                                   void* out, int dtype, int rows, int heads, int kv_heads, int dim, int vdim, int window, int chunk,
+                                   float softcap, int gate_head, void* stream)
+{
+    EXL2_REQUIRE(chunk >= 0 && (chunk == 0 || pool == 0), "window_attn: a chunked mask has no pooled blocks");
+    EXL2_REQUIRE(softcap >= 0.0f, "window_attn: negative soft cap");
     EXL2_REQUIRE(q && k_cache && v_cache && row_seq && row_pos && block_table && out, "window_attn: null operand");
     EXL2_REQUIRE(dtype == 0 || dtype == 1, "window_attn: dtype must be 0 (bfloat16) or 1 (float32)");
     EXL2_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0, "window_attn: bad head shape");
@@ -1000,6 +1064,7 @@ extern "C" int exl2_window_attn(const void* q, const void* k_cache, const void* 
     a.vfreq = vfreq; a.v_rot = v_rot; a.interleaved = interleaved; a.row_seq = row_seq; a.row_pos = row_pos; a.block_table = block_table;
     a.bt_stride = bt_stride; a.page = page; a.pool = pool; a.per_page = pool > 0 ? (page + pool - 1) / pool : 0; a.out = out;
     a.H = heads; a.G = kv_heads; a.dim = dim; a.vdim = vdim; a.window = window; a.page_shift = a.pool_shift = -1;
+    a.chunk = chunk; a.softcap = softcap; a.gate_head = gate_head;
     const size_t smem = (size_t)(dim + vdim) * 4;
     if (dtype == 0) LAUNCH(window_attn_kernel<u16>, dim3(rows, heads), dim3(256), smem, stream, a);
     else LAUNCH(window_attn_kernel<float>, dim3(rows, heads), dim3(256), smem, stream, a);
@@ -1025,6 +1090,20 @@ extern "C" int exl2_window_attn_tiles(const void* q, const void* k_cache, const 
                                       void* out, const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, float* part_o,
                                       float* part_ml, int nsplit, int heads, int kv_heads, int dim, int vdim, int window, void* stream)
 {
+    return exl2_window_attn_tiles_ex(q, k_cache, v_cache, k_pool, v_pool, sink, gate, ldg, vfreq, v_rot, interleaved, row_seq, row_pos,
+                                     block_table, bt_stride, page, pool, out, tile_row0, tile_rows, tiles, tile_mode, part_o, part_ml,
+                                     nsplit, heads, kv_heads, dim, vdim, window, 0, 0.0f, 0, stream);
+}
+
+extern "C" int exl2_window_attn_tiles_ex(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
+                                         const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
+                                         const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
+                                         void* out, const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, float* part_o,
+                                         float* part_ml, int nsplit, int heads, int kv_heads, int dim, int vdim, int window, int chunk,
+                                         float softcap, int gate_head, void* stream)
+{
+    EXL2_REQUIRE(chunk >= 0 && (chunk == 0 || pool == 0), "window_attn_tiles: a chunked mask has no pooled blocks");
+    EXL2_REQUIRE(softcap >= 0.0f, "window_attn_tiles: negative soft cap");
     EXL2_REQUIRE(nsplit >= 1 && nsplit <= 64 && (nsplit == 1 || (tile_mode == 1 && part_o && part_ml)),
                  "window_attn_tiles: key splits (1 .. 64) need tile_mode 1 and scratch");
     EXL2_REQUIRE(q && k_cache && v_cache && row_seq && row_pos && block_table && out && tile_row0, "window_attn_tiles: null operand");
@@ -1033,7 +1112,7 @@ extern "C" int exl2_window_attn_tiles(const void* q, const void* k_cache, const 
     EXL2_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "window_attn_tiles: bad head shape");
     EXL2_REQUIRE(page > 0 && window > 0 && pool >= 0 && (pool == 0 || (k_pool && v_pool)), "window_attn_tiles: bad window / paging");
     EXL2_REQUIRE(!v_rot || vfreq, "window_attn_tiles: rotated values need their frequencies");
-    EXL2_REQUIRE(!gate || (ldg % 4 == 0 && ((uintptr_t)gate % 16) == 0), "window_attn_tiles: gate rows must be 16-byte aligned");
+    EXL2_REQUIRE(!gate || gate_head || (ldg % 4 == 0 && ((uintptr_t)gate % 16) == 0), "window_attn_tiles: gate rows must be 16-byte aligned");
     if (!exl2_window_attn_tiles_supported(dim, vdim))
         EXL2_FAIL(EXL2_E_UNSUPPORTED, "window_attn_tiles: head sizes %d / %d outside the matrix-core form", dim, vdim);
     if (tiles <= 0) return EXL2_OK;
@@ -1043,6 +1122,7 @@ extern "C" int exl2_window_attn_tiles(const void* q, const void* k_cache, const 
     a.vfreq = vfreq; a.v_rot = v_rot; a.interleaved = interleaved; a.row_seq = row_seq; a.row_pos = row_pos; a.block_table = block_table;
     a.bt_stride = bt_stride; a.page = page; a.pool = pool; a.per_page = pool > 0 ? (page + pool - 1) / pool : 0; a.out = out;
     a.H = heads; a.G = kv_heads; a.dim = dim; a.vdim = vdim; a.window = window;
+    a.chunk = chunk; a.softcap = softcap; a.gate_head = gate_head;
     a.page_shift = wa_log2_exact(page); a.pool_shift = pool > 0 ? wa_log2_exact(pool) : -1;
     m.tile_row0 = tile_row0; m.tile_rows = tile_rows; m.part_o = part_o; m.part_ml = part_ml; m.nsplit = nsplit;
     hipStream_t s = (hipStream_t)stream;

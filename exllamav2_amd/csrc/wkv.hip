@@ -1,0 +1,225 @@
+// wkv.hip -- a linear-attention mixer with a per-channel, data-dependent decay (RWKV-style time mixing) for gfx950, + its C ABI.
+//
+// Per head, with r, k (key channels i = 0 .. N) and v (value channels j = 0 .. P) of the token, a decay w_i in (0, 1) and a bonus u_i
+// that only the current token gets, the state S (N x P, fp32) gives
+//     o_j = sum_i r_i (S_ij + u_i k_i v_j),        S_ij <- w_i S_ij + k_i v_j,
+// the head's o is divided by its root mean square, multiplied by a weight per channel and by the gate silu(g), and leaves in the
+// operand dtype for the output projection.  The decay comes as d = log(-log w) (w = exp(-exp(d)), evaluated here in fp32).
+//
+// The five projections read five blends of the mixer's input h with the previous token's input h':  h + (h' - h) * mu_s.
+// wkv_mix_kernel makes them from the fp32 input rows: h' is the row in front when that belongs to the same sequence, else what the
+// sequence's slot keeps, zeros at position 0.
+//
+// Rows of a step are a flat list; a span is the run of consecutive rows one sequence brings (span i = rows span_row0[i] ..
+// + span_rows[i], slot and first position = row_seq / row_pos of its first row).  A span at position 0 starts from zeros whatever
+// its slot holds.  Everything here is fp32 except the operand-dtype outputs.
+#include "hw.h"
+#include "errors.h"
+#include <stdint.h>
+
+template <typename T> DEV float wk_ld(const T* p);
+template <> DEV float wk_ld<u16>(const u16* p) { return bf16_to_f32(*p); }
+template <> DEV float wk_ld<float>(const float* p) { return *p; }
+template <typename T> DEV void wk_st(T* p, float v);
+template <> DEV void wk_st<u16>(u16* p, float v) { *p = f32_to_bf16(v); }
+template <> DEV void wk_st<float>(float* p, float v) { *p = v; }
+
+extern "C" int exl2_span_last_rows(const float* src, int ld, float* slot_rows, int width, const int* span_row0, const int* span_rows,
+                                   int spans, const int* row_seq, void* stream);
+
+// ---- the blends -------------------------------------------------------------------------------------------------------------------
+
+struct MixArgs
+{
+    const float* h; int width;               // [rows, width]
+    float* prev;                             // [slots, width]
+    const void* mu; int n_mix;               // [n_mix, width] operand dtype
+    void* out; long long out_stride;         // blend s at out + s * out_stride: [rows, width] operand dtype
+    const int* row_seq; const int* row_pos;
+    int fused;                               // single-row spans: the slot is rolled here
+};
+
+// grid (rows, width / 256)
+template <typename T>
+KERNEL void __launch_bounds__(256) wkv_mix_kernel(const MixArgs a)
+{
+    const int r = bid_x(), i = bid_y() * 256 + tid();
+    if (i >= a.width) return;
+    const int pos = a.row_pos[r], sq = a.row_seq[r];
+    const float hv = a.h[(long long)r * a.width + i];
+    float hp = 0.0f;
+    if (pos > 0) hp = (!a.fused && r > 0 && a.row_seq[r - 1] == sq) ? a.h[(long long)(r - 1) * a.width + i] : a.prev[(long long)sq * a.width + i];
+    if (a.fused) a.prev[(long long)sq * a.width + i] = hv;
+    const float d = hp - hv;
+    for (int s = 0; s < a.n_mix; s++)
+        wk_st<T>((T*)a.out + s * a.out_stride + (long long)r * a.width + i, fmaf(d, wk_ld<T>((const T*)a.mu + (long long)s * a.width + i), hv));
+}
+
+// ---- the recurrence, token by token ---------------------------------------------------------------------------------------------------
+
+#define WKV_CHUNK 16                         // tokens staged in LDS per round
+#define WKV_MAX_NPT 128                      // state rows per thread
+
+struct WkvArgs
+{
+    const float* r; const float* k; const float* v; const float* g; int ld;      // [rows, ld] each: head h at h * N (r, k) or h * P (v, g)
+    const float* dlog; int ldd;              // [rows, ldd]: log(-log w), head h at h * N
+    const float* u;                          // [heads, N]
+    const float* norm_w;                     // [heads * P]
+    void* out; int ldo;                      // [rows, ldo] operand dtype (or fp32)
+    float* state;                            // [slots, heads, N, P]
+    const int* span_row0; const int* span_rows; const int* row_seq; const int* row_pos;
+    int heads, N, P, KS;                     // KS = threads that share a column of the state (blockDim = P * KS rounded up to waves)
+    float eps;
+};
+
+// Workgroup = one (span, head): thread (j, p) holds rows n = j, j + KS, .. of column p of the state in registers for the whole span.
+// Tokens are taken WKV_CHUNK at a time: r, k, the decay and v are staged in LDS, every thread steps its rows through the chunk keeping
+// one partial sum per token, the KS partial sums of a column are added at the chunk's end, and a wave per token takes the head's
+// root mean square and writes the normed, gated row.
+template <typename T, int NPT>
+KERNEL void __launch_bounds__(256) wkv_scan_kernel(const WkvArgs a)
+{
+    DYN_SMEM(smem);
+    const int h = bid_x(), sp = bid_y();
+    const int n_tok = a.span_rows[sp], r0 = a.span_row0[sp];
+    const int pos0 = a.row_pos[r0];
+    const int P = a.P, N = a.N, KS = a.KS;
+    const int t = tid(), nt = nthreads();
+    const bool owner = t < P * KS;
+    const int p = t % P, j = t / P;
+    float* s_r = (float*)smem;                                   // [CHUNK, N]
+    float* s_k = s_r + WKV_CHUNK * N;                            // [CHUNK, N]
+    float* s_w = s_k + WKV_CHUNK * N;                            // [CHUNK, N]
+    float* s_v = s_w + WKV_CHUNK * N;                            // [CHUNK, P]
+    float* s_o = s_v + WKV_CHUNK * P;                            // [CHUNK, P]
+    float* s_part = s_o + WKV_CHUNK * P;                         // [CHUNK, KS, P]
+    float* st = a.state + ((long long)a.row_seq[r0] * a.heads + h) * (long long)N * P;
+    float S[NPT], U[NPT];
+    #pragma unroll
+    for (int i = 0; i < NPT; i++)
+    {
+        const int n = j + KS * i;
+        S[i] = (owner && pos0 > 0 && n < N) ? st[(long long)n * P + p] : 0.0f;
+        U[i] = n < N ? a.u[h * N + n] : 0.0f;
+    }
+    for (int c0 = 0; c0 < n_tok; c0 += WKV_CHUNK)
+    {
+        const int nc = min(WKV_CHUNK, n_tok - c0);
+        block_sync();
+        for (int i = t; i < nc * N; i += nt)
+        {
+            const long long row = r0 + c0 + i / N;
+            const int n = i % N;
+            s_r[i] = a.r[row * a.ld + h * N + n];
+            s_k[i] = a.k[row * a.ld + h * N + n];
+            s_w[i] = expf(-expf(a.dlog[row * a.ldd + h * N + n]));
+        }
+        for (int i = t; i < nc * P; i += nt) s_v[i] = a.v[(long long)(r0 + c0 + i / P) * a.ld + h * P + i % P];
+        block_sync();
+        for (int kk = 0; owner && kk < nc; kk++)
+        {
+            const float vv = s_v[kk * P + p];
+            float part = 0.0f;
+            #pragma unroll
+            for (int i = 0; i < NPT; i++)
+            {
+                const int n = j + KS * i;
+                if (n < N)
+                {
+                    const float kv = s_k[kk * N + n] * vv;
+                    part = fmaf(s_r[kk * N + n], fmaf(U[i], kv, S[i]), part);
+                    S[i] = fmaf(s_w[kk * N + n], S[i], kv);
+                }
+            }
+            s_part[(kk * KS + j) * P + p] = part;
+        }
+        block_sync();
+        for (int i = t; i < nc * P; i += nt)
+        {
+            const int kk = i / P, pp = i % P;
+            float ov = 0.0f;
+            for (int jj = 0; jj < KS; jj++) ov += s_part[(kk * KS + jj) * P + pp];
+            s_o[i] = ov;
+        }
+        block_sync();
+        for (int kk = wave_id(); kk < nc; kk += nt / 64)
+        {
+            float ss = 0.0f;
+            for (int pp = lane_id(); pp < P; pp += 64) { const float ov = s_o[kk * P + pp]; ss = fmaf(ov, ov, ss); }
+            ss = wave_allreduce_add(ss);
+            const float rinv = 1.0f / sqrtf(ss / (float)P + a.eps);
+            const long long row = r0 + c0 + kk;
+            for (int pp = lane_id(); pp < P; pp += 64)
+            {
+                const float gv = a.g[row * a.ld + h * P + pp];
+                const float o = s_o[kk * P + pp] * rinv * a.norm_w[h * P + pp] * (gv / (1.0f + expf(-gv)));
+                wk_st<T>((T*)a.out + row * a.ldo + h * P + pp, o);
+            }
+        }
+    }
+    #pragma unroll
+    for (int i = 0; i < NPT; i++)
+    {
+        const int n = j + KS * i;
+        if (owner && n < N) st[(long long)n * P + p] = S[i];
+    }
+}
+
+// ---- C ABI ----------------------------------------------------------------------------------------------------------------------
+
+extern "C" int exl2_wkv_mix(const float* h, float* prev, const void* mu, int n_mix, void* out, long long out_stride, const int* row_seq,
+                            const int* row_pos, const int* span_row0, const int* span_rows, int spans, int max_span_rows, int dtype,
+                            int rows, int width, void* stream)
+{
+    EXL2_REQUIRE(h && prev && mu && out && row_seq && row_pos && span_row0 && span_rows, "wkv_mix: null operand");
+    EXL2_REQUIRE(dtype == 0 || dtype == 1, "wkv_mix: dtype must be 0 (bfloat16) or 1 (float32)");
+    EXL2_REQUIRE(n_mix > 0 && width > 0 && out_stride >= (long long)rows * width, "wkv_mix: bad shape");
+    if (rows <= 0 || spans <= 0) return EXL2_OK;
+    MixArgs a;
+    a.h = h; a.width = width; a.prev = prev; a.mu = mu; a.n_mix = n_mix; a.out = out; a.out_stride = out_stride; a.row_seq = row_seq;
+    a.row_pos = row_pos; a.fused = max_span_rows == 1;
+    const dim3 grid(rows, (width + 255) / 256);
+    if (dtype == 0) LAUNCH(wkv_mix_kernel<u16>, grid, dim3(256), 0, stream, a);
+    else LAUNCH(wkv_mix_kernel<float>, grid, dim3(256), 0, stream, a);
+    HIP_TRY(hipGetLastError());
+    if (!a.fused) return exl2_span_last_rows(h, width, prev, width, span_row0, span_rows, spans, row_seq, stream);
+    return EXL2_OK;
+}
+
+template <typename T>
+static void wkv_scan_launch(const WkvArgs& a, int npt, dim3 grid, dim3 block, size_t smem, void* stream)
+{
+    if (npt <= 8) LAUNCH((wkv_scan_kernel<T, 8>), grid, block, smem, stream, a);
+    else if (npt <= 16) LAUNCH((wkv_scan_kernel<T, 16>), grid, block, smem, stream, a);
+    else if (npt <= 32) LAUNCH((wkv_scan_kernel<T, 32>), grid, block, smem, stream, a);
+    else if (npt <= 64) LAUNCH((wkv_scan_kernel<T, 64>), grid, block, smem, stream, a);
+    else LAUNCH((wkv_scan_kernel<T, WKV_MAX_NPT>), grid, block, smem, stream, a);
+}
+
+extern "C" int exl2_wkv_scan(const float* r, const float* k, const float* v, const float* g, int ld, const float* dlog, int ldd,
+                             const float* u, const float* norm_w, void* out, int ldo, int out_f32, float* state,
+                             const int* span_row0, const int* span_rows, int spans, const int* row_seq, const int* row_pos,
+                             int heads, int n_key, int n_val, float eps, void* stream)
+{
+    EXL2_REQUIRE(r && k && v && g && dlog && u && norm_w && out && state && span_row0 && span_rows && row_seq && row_pos,
+                 "wkv_scan: null operand");
+    EXL2_REQUIRE(heads > 0 && n_key > 0 && n_val > 0 && n_val <= 256, "wkv_scan: state %d x %d", n_key, n_val);
+    if (spans <= 0) return EXL2_OK;
+    int ks = 256 / n_val;
+    if (ks < 1) ks = 1;
+    if (ks > n_key) ks = n_key;
+    const int npt = (n_key + ks - 1) / ks;
+    EXL2_REQUIRE(npt <= WKV_MAX_NPT, "wkv_scan: state %d x %d needs %d rows per thread (at most %d)", n_key, n_val, npt, WKV_MAX_NPT);
+    WkvArgs a;
+    a.r = r; a.k = k; a.v = v; a.g = g; a.ld = ld; a.dlog = dlog; a.ldd = ldd; a.u = u; a.norm_w = norm_w; a.out = out; a.ldo = ldo;
+    a.state = state; a.span_row0 = span_row0; a.span_rows = span_rows; a.row_seq = row_seq; a.row_pos = row_pos;
+    a.heads = heads; a.N = n_key; a.P = n_val; a.KS = ks; a.eps = eps;
+    const size_t smem = sizeof(float) * ((size_t)WKV_CHUNK * (3 * n_key + 2 * n_val + (size_t)ks * n_val));
+    EXL2_REQUIRE(smem <= 64 * 1024, "wkv_scan: state %d x %d does not fit the staging buffers", n_key, n_val);
+    const dim3 grid(heads, spans), block((n_val * ks + 63) / 64 * 64);
+    if (out_f32) wkv_scan_launch<float>(a, npt, grid, block, smem, stream);
+    else wkv_scan_launch<u16>(a, npt, grid, block, smem, stream);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}

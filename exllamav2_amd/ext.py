@@ -778,6 +778,7 @@ class ExtC:
     # ---- unquantized models: dense linears, row-wise steps, latent attention (csrc/dense.hip, rowops.hip, latent_attn.hip) ------
 
     EPI_NONE, EPI_MUL_SIGMOID_AUX, EPI_SILU_AUX_MUL, EPI_CLAMPED_GLU, EPI_RELU_SQUARED, EPI_SOFT_CAP = 0, 1, 2, 3, 4, 5
+    EPI_SCALE, EPI_TANH, EPI_ROW_SCALED_RELU_SQUARED = 6, 7, 8        # acc * limit; tanh(acc); relu(aux[row] * acc)^2
 
     @staticmethod
     def _dense_code(dtype) -> int:
@@ -953,47 +954,97 @@ class ExtC:
     def kv_rot_append(self, f, ld: int, q_off: int, k_off: int, v_off: int, q_out, q_scale, k_cache, v_cache, k_pool, v_pool, freq,
                       amp: float, rot_dims: int, vfreq, v_rot: bool, interleaved: bool, row_seq, row_pos, block_table, page: int, pool: int,
                       rows: int, heads: int, kv_heads: int, dim: int, vdim: int) -> None:
-        dt = k_cache.dtype
-        self.lib.check(self.lib.exl2_kv_rot_append(
+        dt = q_out.dtype                                         # (k_cache None: the rows bring queries only)
+        self.lib.check(self.lib.exl2_kv_rot_append_ex(
             self._ptr(f, torch.float32, "f"), int(ld), int(q_off), int(k_off), int(v_off), self._ptr(q_out, dt, "q_out"),
             self._ptr(q_scale, torch.float32, "q_scale"), self._ptr(k_cache, dt, "k_cache"), self._ptr(v_cache, dt, "v_cache"),
             self._ptr(k_pool, dt, "k_pool"), self._ptr(v_pool, dt, "v_pool"), self._ptr(freq, torch.float32, "freq"), float(amp),
             int(rot_dims), self._ptr(vfreq, torch.float32, "vfreq"), int(v_rot), int(interleaved),
             self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
             self._ptr(block_table, torch.int32, "block_table"), block_table.shape[-1], int(page), int(pool), self._dense_code(dt),
-            int(rows), int(heads), int(kv_heads), int(dim), int(vdim), self._stream(k_cache)))
+            int(rows), int(heads), int(kv_heads), int(dim), int(vdim), self._stream(q_out)))
 
     def window_attn(self, q, k_cache, v_cache, k_pool, v_pool, sink, gate, ldg: int, gate_off: int, vfreq, v_rot: bool, interleaved: bool,
                     row_seq, row_pos, block_table, page: int, pool: int, out, rows: int, heads: int, kv_heads: int, dim: int, vdim: int,
-                    window: int) -> None:
+                    window: int, chunk: int = 0, softcap: float = 0.0, gate_head: bool = False) -> None:
+        """chunk > 0: chunked mask instead of the window; softcap > 0: capped scores; gate_head: one gate value per head"""
         dt = k_cache.dtype
         gp = None if gate is None else self._ptr(gate, torch.float32, "gate") + gate_off * 4
-        self.lib.check(self.lib.exl2_window_attn(
+        self.lib.check(self.lib.exl2_window_attn_ex(
             self._ptr(q, dt, "q"), self._ptr(k_cache, dt, "k_cache"), self._ptr(v_cache, dt, "v_cache"), self._ptr(k_pool, dt, "k_pool"),
             self._ptr(v_pool, dt, "v_pool"), self._ptr(sink, torch.float32, "sink"), gp, int(ldg), self._ptr(vfreq, torch.float32, "vfreq"),
             int(v_rot), int(interleaved), self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
             self._ptr(block_table, torch.int32, "block_table"), block_table.shape[-1], int(page), int(pool), self._ptr(out, dt, "out"),
-            self._dense_code(dt), int(rows), int(heads), int(kv_heads), int(dim), int(vdim), int(window), self._stream(out)))
+            self._dense_code(dt), int(rows), int(heads), int(kv_heads), int(dim), int(vdim), int(window), int(chunk), float(softcap),
+            int(gate_head), self._stream(out)))
 
     def window_attn_tiles_supported(self, dtype, dim: int, vdim: int) -> bool:
         return dtype is torch.bfloat16 and bool(self.lib.exl2_window_attn_tiles_supported(int(dim), int(vdim)))
 
     def window_attn_tiles(self, q, k_cache, v_cache, k_pool, v_pool, sink, gate, ldg: int, gate_off: int, vfreq, v_rot: bool,
                           interleaved: bool, row_seq, row_pos, block_table, page: int, pool: int, out, tiles, tile_mode: int, heads: int,
-                          kv_heads: int, dim: int, vdim: int, window: int, nsplit: int = 1, part_o=None, part_ml=None) -> None:
+                          kv_heads: int, dim: int, vdim: int, window: int, nsplit: int = 1, part_o=None, part_ml=None, chunk: int = 0,
+                          softcap: float = 0.0, gate_head: bool = False) -> None:
         """tile_mode 64: tiles = (tile_row0 int32 [n], tile_rows int32 [n], n), runs of <= 64 consecutive positions of one sequence;
         tile_mode 1: tiles = (rows int32 [n], None, n), single decoded rows"""
         row0, nrows, n = tiles
         bf = torch.bfloat16
         gp = None if gate is None else self._ptr(gate, torch.float32, "gate") + gate_off * 4
-        self.lib.check(self.lib.exl2_window_attn_tiles(
+        self.lib.check(self.lib.exl2_window_attn_tiles_ex(
             self._ptr(q, bf, "q"), self._ptr(k_cache, bf, "k_cache"), self._ptr(v_cache, bf, "v_cache"), self._ptr(k_pool, bf, "k_pool"),
             self._ptr(v_pool, bf, "v_pool"), self._ptr(sink, torch.float32, "sink"), gp, int(ldg), self._ptr(vfreq, torch.float32, "vfreq"),
             int(v_rot), int(interleaved), self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
             self._ptr(block_table, torch.int32, "block_table"), block_table.shape[-1], int(page), int(pool), self._ptr(out, bf, "out"),
             self._ptr(row0, torch.int32, "tile_row0"), self._ptr(nrows, torch.int32, "tile_rows"), int(n), int(tile_mode),
             self._ptr(part_o, torch.float32, "part_o"), self._ptr(part_ml, torch.float32, "part_ml"), int(nsplit), int(heads),
-            int(kv_heads), int(dim), int(vdim), int(window), self._stream(out)))
+            int(kv_heads), int(dim), int(vdim), int(window), int(chunk), float(softcap), int(gate_head), self._stream(out)))
+
+    # ---- scalar-gain RMS norm + token shift, sigmoid router (csrc/rowops.hip); decaying linear attention (csrc/wkv.hip) ----------------
+
+    def add_rms_shift(self, x32, y, out, rows: int, gain: float, eps: float, moe_y=None, top: int = 0, shift=None, prev=None, hn=None,
+                      row_seq=None, row_pos=None, spans=None, row_idx=None, dtype=None) -> None:
+        """x32 += y + sum of the row's `top` expert outputs (both optional); out = rms_norm(x32) * gain, shifted towards the previous
+        token's normed row when `shift` is given (prev fp32 [slots, width] keeps it between steps; spans = (row0, rows, n, longest))"""
+        width = x32.shape[-1]
+        dt = dtype if dtype is not None else (shift.dtype if shift is not None else (out.dtype if out is not None else torch.float32))
+        row0, nrows, n, longest = spans if spans is not None else (None, None, 0, 0)
+        self.lib.check(self.lib.exl2_add_rms_shift(
+            self._ptr(x32, torch.float32, "x32"), self._ptr(y, torch.float32, "y"), self._ptr(moe_y, torch.float32, "moe_y"), int(top),
+            float(gain), float(eps), self._ptr(shift, None, "shift"), self._ptr(prev, torch.float32, "prev"),
+            self._ptr(hn, torch.float32, "hn"), self._ptr(out, None, "out"), int(out is not None and out.dtype is torch.float32),
+            self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"), self._ptr(row_idx, torch.int32, "row_idx"),
+            self._ptr(row0, torch.int32, "span_row0"), self._ptr(nrows, torch.int32, "span_rows"), int(n), int(longest),
+            self._dense_code(dt), int(rows), int(width), self._stream(x32)))
+
+    def moe_route_sigmoid(self, logits, ids, wts, rows: int, n_total: int, top: int, scale: float = 1.0, groups=None) -> None:
+        gc, go, gr = groups if groups is not None else (None, None, None)
+        self.lib.check(self.lib.exl2_moe_route_sigmoid(self._ptr(logits, torch.float32, "logits"), self._ptr(ids, torch.int32, "ids"),
+                                                       self._ptr(wts, torch.float32, "wts"), int(rows), int(n_total), int(top), float(scale),
+                                                       self._ptr(gc, torch.int32, "grp_count"), self._ptr(go, torch.int32, "grp_offset"),
+                                                       self._ptr(gr, torch.int32, "grp_rows"), self._stream(logits)))
+
+    def wkv_mix(self, h, prev, mu, out, row_seq, row_pos, spans, rows: int, width: int) -> None:
+        """out[s] = h + (h' - h) * mu[s]; h fp32 [rows, width], mu [n_mix, width] and out [n_mix, rows, width] in the operand dtype"""
+        row0, nrows, n, longest = spans
+        self.lib.check(self.lib.exl2_wkv_mix(self._ptr(h, torch.float32, "h"), self._ptr(prev, torch.float32, "prev"), self._ptr(mu, None, "mu"),
+                                             mu.shape[0], self._ptr(out, mu.dtype, "out"), int(rows) * int(width),
+                                             self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"),
+                                             self._ptr(row0, torch.int32, "span_row0"), self._ptr(nrows, torch.int32, "span_rows"), int(n),
+                                             int(longest), self._dense_code(mu.dtype), int(rows), int(width), self._stream(out)))
+
+    def wkv_scan(self, rkvg, rows: int, dlog, u, norm_w, out, state, spans, row_seq, row_pos, heads: int, n_key: int, n_val: int,
+                 eps: float) -> None:
+        """rkvg fp32 [4, rows, heads * n] (r, k, v, g; n_key == n_val); dlog fp32 [rows, heads * n_key]; out [rows, heads * n_val]"""
+        row0, nrows, n, _longest = spans
+        p = self._ptr(rkvg, torch.float32, "rkvg")
+        step = int(rows) * heads * n_key * 4
+        self.lib.check(self.lib.exl2_wkv_scan(p, p + step, p + 2 * step, p + 3 * step, heads * n_key, self._ptr(dlog, torch.float32, "dlog"),
+                                              dlog.shape[-1], self._ptr(u, torch.float32, "u"), self._ptr(norm_w, torch.float32, "norm_w"),
+                                              self._ptr(out, None, "out"), out.shape[-1], int(out.dtype is torch.float32),
+                                              self._ptr(state, torch.float32, "state"), self._ptr(row0, torch.int32, "span_row0"),
+                                              self._ptr(nrows, torch.int32, "span_rows"), int(n), self._ptr(row_seq, torch.int32, "row_seq"),
+                                              self._ptr(row_pos, torch.int32, "row_pos"), int(heads), int(n_key), int(n_val), float(eps),
+                                              self._stream(out)))
 
     def graph_begin_capture(self, stream: int | None) -> None:
         self.lib.check(self.lib.exl2_graph_begin_capture(stream))

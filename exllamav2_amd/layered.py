@@ -1,9 +1,10 @@
 """Config-driven decoder stack over unquantized weights: each layer is a mixer and an optional feed-forward taken from two
 registries, on an fp32 residual stream.  The residual style is the configuration's: post-norm steps
 x <- norm(alpha x + sublayer(x)) (1 + w)  (RMS norm, a `head` matrix), or pre-norm steps  x <- x + sublayer(layer_norm(x))  (weight and
-bias, logits from the embedding table, optional soft cap).  Mixers: latent attention, windowed attention with pooled blocks,
-state-space scan; a stack may mix them -- each keeps what it needs between steps (pages of keys and values, per-slot recurrent
-state) under one page pool.
+bias, logits from the embedding table, optional soft cap), or pre-norm steps with scalar-gain RMS norms and a token shift in front
+of every mixer (a `head` matrix, scaled logits).  Mixers: latent attention, windowed / chunked attention (pooled blocks, sinks, shared
+keys and values), state-space scan, decaying linear attention; a stack may mix them -- each keeps what it needs between steps (pages
+of keys and values, per-slot recurrent state) under one page pool.
 
 The model has ONE forward, `step(batch, cache)`: the rows of a step are a flat list of tokens, each with its sequence slot and
 position, so whole prompts, portions of prompts and single decoded tokens of several requests run through the same launches
@@ -21,10 +22,11 @@ from .dense_linear import DenseLinear
 from .ext import ext_c
 from .latent_attn import LatentAttention
 from .mlp import DenseActMLP, DenseGatedMLP
-from .moe_mlp import ScoredMoEMLP
-from .rmsnorm import PostNorm, PreLayerNorm
+from .moe_mlp import ScoredMoEMLP, SigmoidMoEMLP
+from .rmsnorm import PostNorm, PreLayerNorm, PreShiftRMSNorm
 from .ssm import StateSpaceMixer
 from .window_attn import WindowAttention
+from .wkv import DecayLinearAttention
 
 
 def _latent_attention(model, key, idx, spec):
@@ -38,10 +40,20 @@ def _latent_attention(model, key, idx, spec):
 def _window_attention(model, key, idx, spec):
     m = spec["mixer"]
     mask, rot = m.get("mask") or {}, m.get("rot") or {}
-    return WindowAttention(model, key, idx, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads") or m["heads"]), dim=int(m["dim"]),
-                           vdim=int(m.get("vdim") or m["dim"]), window=int(mask.get("size") or (1 << 30)), pool=int(mask.get("pool") or 0),
-                           rot_base=float(rot.get("base", 10000.0)), rot_dims=int(rot.get("dims", 0)), rot_scaling=rot.get("scaling"),
-                           scale=float(m["scale"]))
+    common = dict(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads") or m["heads"]), dim=int(m["dim"]), vdim=int(m.get("vdim") or m["dim"]),
+                  rot_base=float(rot.get("base", 10000.0)), rot_dims=int(rot.get("dims", 0)), rot_scaling=rot.get("scaling"),
+                  scale=float(m["scale"]))
+    if model.config.attention_mask == "chunk":
+        # chunks from position 0, capped scores, a constant 1 in the softmax denominator, values as they are, maybe another layer's rows
+        return WindowAttention(model, key, idx, window=1 << 30, pool=0, chunk=int(mask.get("size") or 0), softcap=float(m.get("softcap") or 0.0),
+                               sink_one=True, rotate_values=False, kv_from=(int(m["kv_from"]) if m.get("kv_from") is not None else None),
+                               **common)
+    return WindowAttention(model, key, idx, window=int(mask.get("size") or (1 << 30)), pool=int(mask.get("pool") or 0), **common)
+
+
+def _decay_linear_attention(model, key, idx, spec):
+    m = spec["mixer"]
+    return DecayLinearAttention(model, key, idx, heads=int(m["heads"]), dim=int(m["dim"]))
 
 
 def _state_space(model, key, idx, spec):
@@ -58,12 +70,16 @@ def _dense_mlp(model, key, idx, spec):
 
 def _moe_mlp(model, key, idx, spec):
     r, e = spec["router"], spec["expert"]
+    if model.config.residual == "pre_rms_shift":              # sigmoid scores weigh the experts' inputs; a shared expert beside them
+        shared = spec.get("shared")
+        return SigmoidMoEMLP(model, key, idx, experts=int(r["experts"]), top=int(r["top"]), ff=int(e["ff"]),
+                             shared_ff=(int(shared["ff"]) if shared else None), route_scale=float(r.get("scale", 1.0)))
     return ScoredMoEMLP(model, key, idx, experts=int(r["experts"]), identity=int(r.get("identity", 0)), top=int(r["top"]),
                         route_scale=float(r["scale"]), ff=int(e["ff"]), limit=float(e["limit"]))
 
 
 # config `type` -> builder(model, key, layer index, layer spec)
-MIXERS = {"latent_attention": _latent_attention, "attention": _window_attention, "mamba2": _state_space}
+MIXERS = {"latent_attention": _latent_attention, "attention": _window_attention, "mamba2": _state_space, "wkv": _decay_linear_attention}
 FEED_FORWARDS = {"dense": _dense_mlp, "moe": _moe_mlp}       # config `mlp.kind` -> builder(model, key, layer index, mlp spec)
 
 
@@ -133,17 +149,21 @@ class LayeredModel:
         cfg = self.config
         conv = lambda t: t.to(self.dtype).contiguous() if t.is_floating_point() else t
 
-        def need(name):
+        def need(name, optional=False):
             if name not in tensors:
+                if optional:
+                    return None
                 raise RuntimeError(f"checkpoint has no tensor '{name}'")
             return conv(tensors[name])
 
         self.embed = need("embed")
         if tuple(self.embed.shape) != (cfg.vocab, cfg.width):
             raise RuntimeError(f"embed is {tuple(self.embed.shape)}, config says {(cfg.vocab, cfg.width)}")
-        pre = cfg.residual == "pre_ln"
+        pre = cfg.residual in ("pre_ln", "pre_rms_shift")
 
-        def make_norm(name):
+        def make_norm(name, shift=None):
+            if cfg.residual == "pre_rms_shift":
+                return PreShiftRMSNorm(self.ext, name, need(name), cfg.norm_eps, shift=need(shift) if shift else None)
             if pre:
                 return PreLayerNorm(self.ext, name, need(name), need(name + ".b") if name + ".b" in tensors else None, cfg.norm_eps)
             return PostNorm(self.ext, name, need(name), cfg.norm_eps, cfg.postln_alpha)
@@ -153,8 +173,8 @@ class LayeredModel:
             key = f"l{i}"
             if spec["type"] not in MIXERS:
                 raise RuntimeError(f"layer {i}: unknown mixer type '{spec['type']}' (known: {sorted(MIXERS)})")
-            mixer = MIXERS[spec["type"]](self, key, i, spec).load(lambda n, k=key: need(f"{k}.mix.{n}"))
-            norm1 = make_norm(key + ".norm1")
+            mixer = MIXERS[spec["type"]](self, key, i, spec).load(lambda n, optional=False, k=key: need(f"{k}.mix.{n}", optional))
+            norm1 = make_norm(key + ".norm1", shift=(key + ".shift") if cfg.residual == "pre_rms_shift" else None)
             ff, norm2 = None, None
             ms = spec.get("mlp")
             if ms is not None:
@@ -170,16 +190,20 @@ class LayeredModel:
                 if not (0 <= j < len(self.layers)) or getattr(self.layers[j][0], "kv_from", 0) is not None:
                     raise RuntimeError(f"layer {i}: kv_from {j} does not name a layer with keys and values of its own")
                 src = self.layers[j][0]
-                if (src.kv_rank, src.rot_dim, src.rot_dims, src.rot_base) != (mixer.kv_rank, mixer.rot_dim, mixer.rot_dims, mixer.rot_base):
+                if hasattr(mixer, "check_kv_source"):
+                    if j >= i:
+                        raise RuntimeError(f"layer {i}: kv_from {j} must name an earlier layer (its rows of the step are cached first)")
+                    mixer.check_kv_source(src)
+                elif (src.kv_rank, src.rot_dim, src.rot_dims, src.rot_base) != (mixer.kv_rank, mixer.rot_dim, mixer.rot_dims, mixer.rot_base):
                     raise RuntimeError(f"layer {i}: its latent sizes / rotation differ from layer {j}'s, whose cache it reads")
         if pre:
             self.final_norm = make_norm("final.norm")
             # the sublayers in order, each with the norm in front of it: (norm, module, is a mixer)
             self.sublayers = []
-            for mixer, norm1, ff, norm2 in self.layers:
-                self.sublayers.append((norm1, mixer, True))
+            for i, (mixer, norm1, ff, norm2) in enumerate(self.layers):
+                self.sublayers.append((norm1, mixer, True, i))
                 if ff is not None:
-                    self.sublayers.append((norm2, ff, False))
+                    self.sublayers.append((norm2, ff, False, i))
         else:
             self.final_norm = need("final.norm")
         self.head = DenseLinear(self.ext, "head", self.embed if cfg.tied_head else need("head"))
@@ -197,7 +221,9 @@ class LayeredModel:
 
     def make_cache(self, pool: PagePool):
         if any(hasattr(mixer, "make_state") for mixer, *_rest in self.layers):
-            return LayerStates(pool, {i: mixer.make_state(pool, self.dtype) for i, (mixer, *_rest) in enumerate(self.layers)})
+            norm_states = {i: norm1.make_state(pool, self.width) for i, (_m, norm1, *_r) in enumerate(self.layers) if hasattr(norm1, "make_state")}
+            return LayerStates(pool, {i: mixer.make_state(pool, self.dtype) for i, (mixer, *_rest) in enumerate(self.layers)},
+                               norm_states=norm_states)
         widths, owner = {}, {}
         for i, (mixer, *_rest) in enumerate(self.layers):
             if mixer.kv_from is None:
@@ -215,6 +241,8 @@ class LayeredModel:
         ext, cfg, rows = self.ext, self.config, batch.rows
         if cfg.residual == "pre_ln":
             return self._step_pre_norm(batch, cache)
+        if cfg.residual == "pre_rms_shift":
+            return self._step_pre_rms_shift(batch, cache)
         x32 = self.buf("x32", (rows, self.width), torch.float32)
         xh = x32 if self.dtype is torch.float32 else self.buf("xh", (rows, self.width), self.dtype)
         ext.embed_scale(self.embed, batch.ids, x32, xh, cfg.embedding_scale)
@@ -242,7 +270,7 @@ class LayeredModel:
         xh = self.buf("xh", (rows, self.width), self.dtype)
         ext.embed_scale(self.embed, batch.ids, x32, None, cfg.embedding_scale)
         y = None
-        for norm, module, is_mixer in self.sublayers:
+        for norm, module, is_mixer, _layer in self.sublayers:
             norm.forward(x32, y, xh, rows)
             y = module.forward(xh, rows, batch, cache) if is_mixer else module.forward(xh, rows)[0]
         if y is not None:
@@ -254,3 +282,34 @@ class LayeredModel:
         cap = cfg.logit_softcap
         return self.head.forward(xn, batch.n_logits, out=self.buf("logits", (batch.n_logits, self.vocab), torch.float32),
                                  epi=ext.EPI_SOFT_CAP if cap > 0 else ext.EPI_NONE, limit=cap)
+
+    def _step_pre_rms_shift(self, batch: StepBatch, cache) -> torch.Tensor | None:
+        """x <- x + mixer(shift(norm1(x))), x <- x + ff(norm2(x)) with scalar-gain RMS norms: as in the layer-norm stacks every
+        residual addition -- a linear's output, a shared expert's, the chosen experts' rows -- runs in the launch of the norm that
+        follows it, which also shifts the normed rows towards the previous token's (kept per slot) in front of a mixer.  A mixer
+        that blends its input further (`input_f32`) gets fp32 rows.  Logits: head(norm(x)) * logit_scale, for the wanted rows."""
+        ext, cfg, rows, f32 = self.ext, self.config, batch.rows, torch.float32
+        x32 = self.buf("x32", (rows, self.width), f32)
+        xh = self.buf("xh", (rows, self.width), self.dtype)
+        ext.embed_scale(self.embed, batch.ids, x32, None, 1.0)
+        multi = batch.spans_dev[3] > 1                        # spans of several rows: the shift reads the normed rows from a buffer
+        pending = None
+        for norm, module, is_mixer, layer in self.sublayers:
+            if is_mixer:
+                out = self.buf("xh32", (rows, self.width), f32) if getattr(module, "input_f32", False) else xh
+                hn = self.buf("hn", (rows, self.width), f32) if multi else None
+                norm.forward(x32, pending, out, rows, batch=batch, state=cache.norm_state(layer), hn=hn, dtype=self.dtype)
+                pending = (module.forward(out, rows, batch, cache), None, 0)
+            else:
+                norm.forward(x32, pending, xh, rows, dtype=self.dtype)
+                y, mix = module.forward(xh, rows)
+                pending = (y, mix[0], mix[1].shape[-1]) if mix is not None else (y, None, 0)
+        if pending is not None:
+            self.final_norm.forward(x32, pending, None, rows, dtype=self.dtype)
+        if batch.n_logits == 0:
+            return None
+        xn = self.buf("xn", (batch.n_logits, self.width), self.dtype)
+        self.final_norm.forward(x32, None, xn, batch.n_logits, row_idx=batch.logit_rows, dtype=self.dtype)
+        scaled = cfg.logit_scale != 1.0
+        return self.head.forward(xn, batch.n_logits, out=self.buf("logits", (batch.n_logits, self.vocab), f32),
+                                 epi=ext.EPI_SCALE if scaled else ext.EPI_NONE, limit=cfg.logit_scale)

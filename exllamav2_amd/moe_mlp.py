@@ -119,3 +119,64 @@ class ScoredMoEMLP:
                          aux=g, ldaux=ff, epi=ext.EPI_CLAMPED_GLU, limit=self.limit, **kw)
         ext.dense_linear(a, self.down.weight, y, pairs, width, ff, ff, ff, width, swb=width * ff, **kw)
         return None, (y, ids, wts, E)
+
+
+class SigmoidMoEMLP:
+    """Sparse MoE whose router scores every expert on its own: s = sigmoid(W_router h) in fp32, the `top` largest are chosen and
+    weigh their experts as they are (no renormalisation).  The weight multiplies the expert's INPUT: the token's part is
+    sum_e expert_e(s_e h), expert(z) = W_down act(W_up z) with act = relu^2 and no gate matrix; since W_up (s h) = s (W_up h) the
+    up projection runs on h and the weight enters in its epilogue, in front of the activation (csrc/dense.hip).  A shared expert of
+    the same form (its own width) runs for every token.  Few rows: every (token, choice) pair names its expert's slab; many rows:
+    one grouped launch per projection.  forward returns (y | None, mixture): y is the shared expert's output, the chosen experts'
+    rows are added by the residual step's launch (rmsnorm.PreShiftRMSNorm)."""
+
+    PAIR_ROWS_MAX = 64
+
+    def __init__(self, model, key: str, layer_idx: int, *, experts: int, top: int, ff: int, shared_ff: int | None, route_scale: float = 1.0):
+        self.model, self.ext, self.key, self.layer_idx = model, model.ext, key, layer_idx
+        self.experts, self.top, self.ff, self.shared_ff, self.route_scale = experts, top, ff, shared_ff, route_scale
+        if not 0 < top <= experts:
+            raise ValueError(f"{key}: top {top} of {experts} experts")
+
+    def load(self, get):
+        from .dense_linear import DenseLinear
+        from .mlp import DenseActMLP
+        E, width = self.experts, self.model.width
+        self.router = DenseLinear(self.ext, self.key + ".router", get("router"))
+        stack = lambda name: torch.stack([get(f"e{e}.{name}") for e in range(E)], 0)
+        self.up = DenseLinear(self.ext, self.key + ".up", stack("up"))
+        self.down = DenseLinear(self.ext, self.key + ".down", stack("down"))
+        if tuple(self.router.weight.shape) != (E, width) or tuple(self.up.weight.shape) != (E, self.ff, width) \
+                or tuple(self.down.weight.shape) != (E, width, self.ff):
+            raise RuntimeError(f"{self.key}: tensor shapes do not match the feed-forward's sizes")
+        self.shared = None
+        if self.shared_ff:
+            self.shared = DenseActMLP(self.model, self.key + ".shared", self.layer_idx).load(lambda n: get("shared." + n))
+            if self.shared.up.out_features != self.shared_ff:
+                raise RuntimeError(f"{self.key}: the shared expert is {self.shared.up.out_features} wide, config says {self.shared_ff}")
+        return self
+
+    def weight_bytes(self) -> int:
+        n = self.router.weight_bytes() + (self.up.weight_bytes() + self.down.weight_bytes()) // self.experts * self.top
+        return n + (self.shared.weight_bytes() if self.shared is not None else 0)
+
+    def forward(self, xh: torch.Tensor, rows: int):
+        ext, m = self.ext, self.model
+        E, top, ff, width, dt = self.experts, self.top, self.ff, m.width, m.dtype
+        logits = self.router.forward(xh, rows, out=m.buf("moe.logits", (rows, E), torch.float32))
+        ids = m.buf("moe.ids", (rows, top), torch.int32)
+        wts = m.buf("moe.wts", (rows, top), torch.float32)
+        pairs = rows * top
+        grouped = pairs > self.PAIR_ROWS_MAX
+        groups = None
+        if grouped:
+            groups = (m.buf("moe.count", (E,), torch.int32), m.buf("moe.offset", (E,), torch.int32), m.buf("moe.rows", (pairs,), torch.int32))
+        ext.moe_route_sigmoid(logits, ids, wts, rows, E, top, self.route_scale, groups=groups)
+        a = m.buf("moe.a", (pairs, ff), dt)
+        y = m.buf("moe.y", (pairs, width), torch.float32)
+        kw = dict(batch=E, groups=groups) if grouped else dict(w_sel=ids.view(-1), n_sel=E)
+        ext.dense_linear(xh, self.up.weight, a, pairs, ff, width, width, width, ff, swb=ff * width, x_div=top,
+                         aux=wts, ldaux=1, epi=ext.EPI_ROW_SCALED_RELU_SQUARED, **kw)
+        ext.dense_linear(a, self.down.weight, y, pairs, width, ff, ff, ff, width, swb=width * ff, **kw)
+        ys = self.shared.forward(xh, rows)[0] if self.shared is not None else None
+        return ys, (y, ids, wts, E)

@@ -51,3 +51,31 @@ class PreLayerNorm:
 
     def forward(self, x32: torch.Tensor, y, out: torch.Tensor, rows: int, row_idx=None) -> None:
         self.ext.add_layer_norm(x32, y, self.weight, self.bias, out, rows, self.eps, row_idx=row_idx)
+
+
+class PreShiftRMSNorm:
+    """The norm in front of a sublayer of a pre-norm layer whose gain is ONE number: x / sqrt(mean(x^2) + eps) * g, optionally
+    followed by a token shift  h + (h' - h) * shift  towards the previous token's normed row h' (zeros at a sequence's start).
+    Like PreLayerNorm it runs fused with the residual addition of the sublayer before it -- a linear's fp32 output and / or the
+    `top` expert outputs of every row (csrc/rowops.hip: add_rms_shift_kernel).  The previous row is per-sequence state:
+    `make_state` asks the pool for one fp32 row per slot; steps of single tokens shift and roll it inside the norm's launch."""
+
+    def __init__(self, ext, key: str, gain: torch.Tensor, eps: float, shift: torch.Tensor | None = None):
+        if gain.numel() != 1:
+            raise RuntimeError(f"{key}: the gain of this norm is one number, got {tuple(gain.shape)}")
+        self.ext, self.key, self.eps = ext, key, eps
+        self.gain = float(gain.to(torch.float32).reshape(()).item())
+        self.shift = shift.contiguous() if shift is not None else None
+
+    def make_state(self, pool, width: int):
+        from .cache import SlotState
+        return SlotState(pool, {"prev": (width,)}) if self.shift is not None else None
+
+    def forward(self, x32: torch.Tensor, pending, out: torch.Tensor | None, rows: int, batch=None, state=None, hn=None, row_idx=None,
+                dtype=None) -> None:
+        """pending: None or (y fp32 [rows, width] | None, expert outputs fp32 [rows * top, width] | None, top)"""
+        y, moe_y, top = pending if pending is not None else (None, None, 0)
+        kw = {}
+        if self.shift is not None and out is not None:
+            kw = dict(shift=self.shift, prev=state["prev"], hn=hn, row_seq=batch.row_seq, row_pos=batch.row_pos, spans=batch.spans_dev)
+        self.ext.add_rms_shift(x32, y, out, rows, self.gain, self.eps, moe_y=moe_y, top=top, row_idx=row_idx, dtype=dtype, **kw)

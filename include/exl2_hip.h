@@ -514,6 +514,68 @@ int exl2_window_attn_tiles(const void* q, const void* k_cache, const void* v_cac
                            void* out, const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, float* part_o,
                            float* part_ml, int nsplit, int heads, int kv_heads, int dim, int vdim, int window, void* stream);
 
+/* ---- variants of the windowed attention (csrc/window_attn.hip): the same three calls with
+   chunk > 0: a chunked mask instead of the window -- position p sees j <= p with floor(j / chunk) == floor(p / chunk), chunks
+              counted from the sequence's start (pool must be 0);
+   softcap > 0: score <- softcap * tanh(score / softcap) before the softmax;
+   gate_head: gate holds ONE value per head (gate[r * ldg + h]) instead of one per output value;
+   exl2_kv_rot_append_ex with k_cache == v_cache == NULL: the rows bring queries only (a layer that attends over the keys and
+   values another layer cached). */
+int exl2_kv_rot_append_ex(const float* f, int ld, int q_off, int k_off, int v_off, void* q_out, const float* q_scale,
+                          void* k_cache, void* v_cache, void* k_pool, void* v_pool, const float* freq, float amp, int rot_dims,
+                          const float* vfreq, int v_rot, int interleaved, const int* row_seq, const int* row_pos,
+                          const int* block_table, int bt_stride, int page, int pool, int dtype, int rows, int heads,
+                          int kv_heads, int dim, int vdim, void* stream);
+int exl2_window_attn_ex(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
+                        const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
+                        const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
+                        void* out, int dtype, int rows, int heads, int kv_heads, int dim, int vdim, int window, int chunk,
+                        float softcap, int gate_head, void* stream);
+int exl2_window_attn_tiles_ex(const void* q, const void* k_cache, const void* v_cache, const void* k_pool, const void* v_pool,
+                              const float* sink, const float* gate, int ldg, const float* vfreq, int v_rot, int interleaved,
+                              const int* row_seq, const int* row_pos, const int* block_table, int bt_stride, int page, int pool,
+                              void* out, const int* tile_row0, const int* tile_rows, int tiles, int tile_mode, float* part_o,
+                              float* part_ml, int nsplit, int heads, int kv_heads, int dim, int vdim, int window, int chunk,
+                              float softcap, int gate_head, void* stream);
+
+/* ---- pre-norm stacks with a scalar-gain RMS norm and a token shift (csrc/rowops.hip).  Further epilogues of exl2_dense_linear(_bias):
+   6 acc * limit, 7 tanh(acc), 8 relu(aux[row * ldaux] * acc)^2 (ONE aux value per row). */
+
+/* x[r] += y[r] + sum_k moe_y[r * top + k] (both nullable) on the fp32 stream; hn = x / sqrt(mean(x^2) + eps) * gain; without a
+   shift out[r] = hn[r] (row_idx, nullable and without additions: output row r is made from stream row row_idx[r]); with shift
+   (operand dtype [width]) out[r] = hn[r] + (hn' - hn[r]) * shift, hn' = the normed row of the sequence's previous token -- the row in
+   front of r when it belongs to the same sequence, else prev[row_seq[r]] (fp32 [slots, width]), zeros at position 0 -- and
+   afterwards prev holds the normed row of every span's last token.  hn fp32 [rows, width]: scratch, needed when max_span_rows > 1.
+   out in the operand dtype or fp32; out == NULL: only the additions. */
+int exl2_add_rms_shift(float* x, const float* y, const float* moe_y, int top, float gain, float eps, const void* shift,
+                       float* prev, float* hn, void* out, int out_f32, const int* row_seq, const int* row_pos,
+                       const int* row_idx, const int* span_row0, const int* span_rows, int spans, int max_span_rows,
+                       int dtype, int rows, int width, void* stream);
+/* slot_rows[row_seq[last row of span s]] = src[last row of span s, :width] for every span (fp32) */
+int exl2_span_last_rows(const float* src, int ld, float* slot_rows, int width, const int* span_row0, const int* span_rows,
+                        int spans, const int* row_seq, void* stream);
+/* router with independent scores: score = sigmoid(logit); the `top` largest are chosen (first index on a tie); weight = score *
+   scale, not renormalised.  grp_* as in exl2_moe_route_scored. */
+int exl2_moe_route_sigmoid(const float* logits, int* ids, float* wts, int rows, int n_total, int top, float scale,
+                           int* grp_count, int* grp_offset, int* grp_rows, void* stream);
+
+/* ---- linear attention with a per-channel data-dependent decay (csrc/wkv.hip) */
+
+/* out[s][r] = h[r] + (h' - h[r]) * mu[s] for s < n_mix (operand dtype, blend s at out + s * out_stride), h fp32 [rows, width], h' =
+   the previous token's h (the row in front within a span, else prev[slot], zeros at position 0); afterwards prev holds every
+   span's last h. */
+int exl2_wkv_mix(const float* h, float* prev, const void* mu, int n_mix, void* out, long long out_stride, const int* row_seq,
+                 const int* row_pos, const int* span_row0, const int* span_rows, int spans, int max_span_rows, int dtype,
+                 int rows, int width, void* stream);
+/* per head and row, state S fp32 [slots, heads, n_key, n_val]: o_j = sum_i r_i (S_ij + u_i k_i v_j); S_ij <- w_i S_ij + k_i v_j
+   with w = exp(-exp(dlog)); out = o / sqrt(mean_j(o^2) + eps) * norm_w * silu(g).  r, k [rows, ld] head h at h * n_key; v, g at
+   h * n_val; dlog [rows, ldd]; u fp32 [heads, n_key]; norm_w fp32 [heads * n_val]; out [rows, ldo] operand dtype (bfloat16) or fp32.
+   The state is read at a span's start (unless it starts at position 0) and written at its end. */
+int exl2_wkv_scan(const float* r, const float* k, const float* v, const float* g, int ld, const float* dlog, int ldd,
+                  const float* u, const float* norm_w, void* out, int ldo, int out_f32, float* state,
+                  const int* span_row0, const int* span_rows, int spans, const int* row_seq, const int* row_pos,
+                  int heads, int n_key, int n_val, float eps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
