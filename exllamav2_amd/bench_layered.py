@@ -1,7 +1,9 @@
 """Prefill and decode throughput of the layer-stack models at layer sizes of real models (random weights), each beside the closest
 other model of the package at equal size: the latent-attention / scored-MoE stack beside a Mixtral-style EXL2 stack (same width,
 expert width, expert count, depth), the state-space / windowed-attention stack beside a latent-attention stack (same width, depth,
-heads, window, feed-forward parameters).  Used by `bench.py --design benolix | tibalorn`; one JSON object per size and model."""
+heads, window, feed-forward parameters), the token-shifted chunked-attention / linear-attention stack beside a state-space /
+windowed-attention stack (same width, depth, heads, reach, streamed feed-forward parameters).  Used by
+`bench.py --design benolix | tibalorn | negilorn`; one JSON object per size and model."""
 from __future__ import annotations
 
 import json
@@ -273,8 +275,132 @@ def bench_hybrid_peer(size: str, device="cuda:0", prompt: int = 2048, ctx: int =
     return _bench_engine(model, out, s["vocab"], prompt, ctx, decode_steps, batches)
 
 
+SHIFT_SIZES = {
+    # pattern: a = chunked attention, k = the same reading the keys / values of the attention layer before it, w = decaying linear
+    # attention; d / m = the layer before has a dense / sparse feed-forward
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=128, chunk=1024, rot_dims=64, wkv_heads=32, wkv_dim=64, rank=64,
+                  ff=5632, experts=8, top=2, expert_ff=2816, shared_ff=2816, pattern="adwmkdwm", vocab=32000),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, chunk=2048, rot_dims=128, wkv_heads=64, wkv_dim=64, rank=128,
+                  ff=14336, experts=8, top=2, expert_ff=7168, shared_ff=7168, pattern="adwm", vocab=32000),
+}
+
+
+def shift_config(s: dict) -> dict:
+    layers, last_attn = [], None
+    for ch in s["pattern"]:
+        if ch == "d":
+            layers[-1]["mlp"] = {"ff": s["ff"], "kind": "dense"}
+        elif ch == "m":
+            layers[-1]["mlp"] = {"expert": {"ff": s["expert_ff"]}, "kind": "moe", "router": {"experts": s["experts"], "top": s["top"]},
+                                 "shared": {"ff": s["shared_ff"]}}
+        elif ch == "w":
+            layers.append({"type": "wkv", "mlp": None, "mixer": {"dim": s["wkv_dim"], "heads": s["wkv_heads"]}})
+        else:
+            m = {"dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv_heads"], "vdim": s["vdim"], "mask": {"size": s["chunk"]},
+                 "scale": s["dim"] ** -0.5, "softcap": 50.0,
+                 "rot": {"base": 500000.0, "dims": s["rot_dims"], "scaling": {"factor": 8.0, "original": 8192, "low": 1.0, "high": 4.0}}}
+            if ch == "k":
+                m["kv_from"] = last_attn
+            else:
+                last_attn = len(layers)
+            layers.append({"type": "attention", "mlp": None, "mixer": m})
+    return {"architecture": "Negilorn", "layers": layers, "logit_scale": 0.5, "norm": {"eps": 1e-5}, "vocab": s["vocab"], "width": s["width"]}
+
+
+def shift_random_tensors(cfg: dict, s: dict, device, seed: int = 0) -> dict:
+    g = torch.Generator(device=device).manual_seed(seed)
+    T = {}
+
+    def mat(name, out, inp, gain=1.0):
+        T[name] = (torch.randn((out, inp), device=device, generator=g) * gain / inp ** 0.5).to(torch.bfloat16)
+
+    def vec(name, n, centre, spread=0.1):
+        T[name] = (centre + spread * torch.randn((n,), device=device, generator=g)).to(torch.bfloat16)
+
+    def one(name):
+        T[name] = torch.ones((), device=device, dtype=torch.bfloat16)
+
+    w = cfg["width"]
+    T["embed"] = (torch.randn((cfg["vocab"], w), device=device, generator=g) * 0.5).to(torch.bfloat16)
+    mat("head", cfg["vocab"], w); one("final.norm")
+    for i, L in enumerate(cfg["layers"]):
+        m, k = L["mixer"], f"l{i}"
+        one(k + ".norm1"); vec(k + ".shift", w, 0.3)
+        if L["type"] == "wkv":
+            inner = m["heads"] * m["dim"]
+            for n in "rkvgw":
+                vec(f"{k}.mix.mu.{n}", w, 0.5)
+            for n in "rkvg":
+                mat(f"{k}.mix.{n}", inner, w)
+            mat(k + ".mix.w1", s["rank"], w); mat(k + ".mix.w2", inner, s["rank"]); vec(k + ".mix.w0", inner, -1.0, 0.5)
+            T[k + ".mix.u"] = (0.3 * torch.randn((m["heads"], m["dim"]), device=device, generator=g)).to(torch.bfloat16)
+            vec(k + ".mix.norm", inner, 1.0); mat(k + ".mix.o", w, inner)
+        else:
+            H, G, dim, vd = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            mat(k + ".mix.q", H * dim, w)
+            if "kv_from" not in m:
+                mat(k + ".mix.k", G * dim, w); mat(k + ".mix.v", G * vd, w)
+            mat(k + ".mix.g", H, w); mat(k + ".mix.o", w, H * vd)
+        ms = L["mlp"]
+        if ms is not None:
+            one(k + ".norm2")
+            if ms["kind"] == "dense":
+                mat(k + ".mlp.gate", ms["ff"], w); mat(k + ".mlp.up", ms["ff"], w); mat(k + ".mlp.down", w, ms["ff"])
+            else:
+                mat(k + ".mlp.router", ms["router"]["experts"], w)
+                for e in range(ms["router"]["experts"]):
+                    mat(f"{k}.mlp.e{e}.up", ms["expert"]["ff"], w); mat(f"{k}.mlp.e{e}.down", w, ms["expert"]["ff"])
+                mat(k + ".mlp.shared.up", ms["shared"]["ff"], w); mat(k + ".mlp.shared.down", w, ms["shared"]["ff"])
+    return T
+
+
+def bench_shift(size: str, device="cuda:0", prompt: int = 2048, ctx: int = 1024, decode_steps: int = 64, batches=(1, 4)) -> dict:
+    from .config import LayeredConfig
+    from .layered import LayeredModel
+    s = SHIFT_SIZES[size]
+    cfg = shift_config(s)
+    model = LayeredModel(LayeredConfig.from_dict_prerms_shift(cfg), device=device, dtype=torch.bfloat16).load(shift_random_tensors(cfg, s, device))
+    out = {"design": "negilorn", "size": size, "layers": len(cfg["layers"]), "pattern": s["pattern"], "weight_bytes_per_token": model.weight_bytes()}
+    return _bench_engine(model, out, s["vocab"], prompt, ctx, decode_steps, batches)
+
+
+def bench_shift_peer(size: str, device="cuda:0", prompt: int = 2048, ctx: int = 1024, decode_steps: int = 64, batches=(1, 4)) -> dict:
+    """the closest model of the package: a state-space / windowed-attention stack (bfloat16, the same engine) of the same width and
+    depth -- a state-space layer for every linear-attention layer (as many heads of the same size, state 128), a windowed
+    attention layer of the same heads and reach for every chunked one, a two-matrix feed-forward with the parameters a token
+    streams through behind the same layers"""
+    from .config import LayeredConfig
+    from .layered import LayeredModel
+    s = SHIFT_SIZES[size]
+    layers = []
+    for L in shift_config(s)["layers"]:
+        ms = L["mlp"]
+        ff = None
+        if ms is not None:
+            ff = ms["ff"] * 3 // 2 if ms["kind"] == "dense" else s["expert_ff"] * s["top"] + s["shared_ff"]
+        if L["type"] == "wkv":
+            layers.append({"type": "mamba2", "mixer": {"conv": 4, "groups": 8, "heads": s["wkv_heads"], "norm_groups": 8, "state": 128,
+                                                       "vdim": s["wkv_dim"]}, "mlp": {"ff": ff, "kind": "dense"} if ff else None})
+        else:
+            layers.append({"type": "attention", "mlp": {"ff": ff, "kind": "dense"} if ff else None,
+                           "mixer": {"dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv_heads"], "vdim": s["vdim"],
+                                     "mask": {"pool": 64, "size": s["chunk"]}, "scale": s["dim"] ** -0.5,
+                                     "rot": {"base": 500000.0, "dims": s["rot_dims"],
+                                             "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}})
+    cfg = {"architecture": "Tibalorn", "embedding": {"scale": 1.0}, "layers": layers, "logit_softcap": 30.0, "norm": {"eps": 1e-5},
+           "vocab": s["vocab"], "width": s["width"]}
+    model = LayeredModel(LayeredConfig.from_dict_prenorm(cfg), device=device, dtype=torch.bfloat16).load(hybrid_random_tensors(cfg, device))
+    out = {"design": "tibalorn-peer", "size": size, "layers": len(layers), "weight_bytes_per_token": model.weight_bytes()}
+    return _bench_engine(model, out, s["vocab"], prompt, ctx, decode_steps, batches)
+
+
 def run(sizes, device="cuda:0", peer: bool = True, design: str = "benolix"):
     for size in sizes:
+        if design == "negilorn":
+            print(json.dumps(bench_shift(size, device)), flush=True)
+            if peer:
+                print(json.dumps(bench_shift_peer(size, device)), flush=True)
+            continue
         if design == "tibalorn":
             print(json.dumps(bench_hybrid(size, device)), flush=True)
             if peer:
