@@ -137,6 +137,8 @@ PROTOTYPES = {
     "exl2_moe_route_sigmoid": (ci, [vp, vp, vp, ci, ci, ci, cf, vp, vp, vp, vp]),
     "exl2_wkv_mix": (ci, [vp, vp, vp, ci, vp, cll, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]),
     "exl2_wkv_scan": (ci, [vp, vp, vp, vp, ci, vp, ci, vp, vp, vp, ci, ci, vp, vp, vp, ci, vp, vp, ci, ci, ci, cf, vp]),
+    "exl2_wkv_scan_chunked_supported": (ci, [ci, ci]),
+    "exl2_wkv_scan_chunked": (ci, [vp, vp, vp, vp, ci, vp, ci, vp, vp, vp, ci, ci, vp, vp, vp, vp, ci, ci, ci, vp, vp, vp, vp, ci, ci, ci, cf, vp]),
     # graphs
     "exl2_graph_begin_capture": (ci, [vp]),
     "exl2_graph_end_capture": (ci, [vp, C.POINTER(vp)]),

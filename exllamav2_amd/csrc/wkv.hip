@@ -166,6 +166,183 @@ KERNEL void __launch_bounds__(256) wkv_scan_kernel(const WkvArgs a)
     }
 }
 
+// ---- the same recurrence in chunks (portions of prompts) ------------------------------------------------------------------------------
+// Inside a chunk of WKC_L tokens the recurrence unrolls.  With l_t = log w_t = -exp(d_t) (per key channel), c_t = l_1 + .. + l_t and
+// c_0 = 0:
+//     o_t = (r_t * exp(c_{t-1}))^T S_in + sum_{s < t} A_ts v_s + (r_t . (u * k_t)) v_t,   A_ts = sum_i r_t[i] k_s[i] exp(c_{t-1}[i] - c_s[i]),
+//     S_out = diag(exp(c_L)) S_in + sum_s diag(exp(c_L - c_s)) k_s v_s^T.
+// Every exponent is a difference of the running sum taken the right way round (<= 0), evaluated per (t, s, channel): no factor
+// exp(-c_s) that a fast decay would overflow.  Three launches make every (chunk, head) of a step independent work: (1) each chunk's
+// own contribution Z to S_out and its total decay, (2) the carry over a span's chunks, one thread per state element (Z is replaced by
+// the state ENTERING the chunk, the slot takes the state after the last), (3) each chunk's outputs with the head norm and gate.
+
+#define WKC_L 64
+
+struct WkvChunkArgs
+{
+    WkvArgs a;
+    const int* span_chunk0; int spans;       // chunks in front of each span
+    float* zbuf;                             // [chunks, heads, N, P]
+    float* dbuf;                             // [chunks, heads, N]
+};
+
+// chunk c of the step -> its span, first row and row count
+DEV void wkc_locate(const WkvChunkArgs& g, int c, int& sp, int& r0, int& n)
+{
+    sp = 0;
+    for (int i = 1; i < g.spans; i++) if (g.span_chunk0[i] <= c) sp = i;
+    const int first = (c - g.span_chunk0[sp]) * WKC_L;
+    r0 = g.a.span_row0[sp] + first;
+    n = min(WKC_L, g.a.span_rows[sp] - first);
+}
+
+// cc[0] = 0, cc[t + 1] = c_t for the chunk's n tokens (rows of NS floats); all threads call it
+DEV void wkc_log_decay_sums(const WkvArgs& a, int h, int r0, int n, float* cc, int NS)
+{
+    const int N = a.N;
+    for (int i = tid(); i < (n + 1) * N; i += nthreads())
+    {
+        const int t = i / N, ch = i % N;
+        cc[t * NS + ch] = t == 0 ? 0.0f : -expf(a.dlog[(long long)(r0 + t - 1) * a.ldd + h * N + ch]);
+    }
+    block_sync();
+    for (int ch = tid(); ch < N; ch += nthreads())
+    {
+        float run = 0.0f;
+        for (int t = 1; t <= n; t++) { run += cc[t * NS + ch]; cc[t * NS + ch] = run; }
+    }
+    block_sync();
+}
+
+// grid (chunks, heads)
+KERNEL void __launch_bounds__(256) wkv_chunk_state_kernel(const WkvChunkArgs g)
+{
+    DYN_SMEM(smem);
+    const WkvArgs& a = g.a;
+    const int c = bid_x(), h = bid_y(), N = a.N, P = a.P, NS = N + 1;
+    int sp, r0, n;
+    wkc_locate(g, c, sp, r0, n);
+    float* cc = (float*)smem;                                    // [L + 1][NS]
+    float* kd = cc + (WKC_L + 1) * NS;                           // [L][NS]
+    float* sv = kd + WKC_L * NS;                                 // [L][P]
+    wkc_log_decay_sums(a, h, r0, n, cc, NS);
+    for (int i = tid(); i < n * N; i += 256)
+    {
+        const int t = i / N, ch = i % N;
+        kd[t * NS + ch] = expf(cc[n * NS + ch] - cc[(t + 1) * NS + ch]) * a.k[(long long)(r0 + t) * a.ld + h * N + ch];
+    }
+    for (int i = tid(); i < n * P; i += 256) sv[i] = a.v[(long long)(r0 + i / P) * a.ld + h * P + i % P];
+    block_sync();
+    float* z = g.zbuf + ((long long)c * a.heads + h) * N * P;
+    for (int e = tid(); e < N * P; e += 256)
+    {
+        const int ch = e / P, j = e % P;
+        float acc = 0.0f;
+        for (int t = 0; t < n; t++) acc = fmaf(kd[t * NS + ch], sv[t * P + j], acc);
+        z[e] = acc;
+    }
+    for (int ch = tid(); ch < N; ch += 256) g.dbuf[((long long)c * a.heads + h) * N + ch] = expf(cc[n * NS + ch]);
+}
+
+// grid (spans, heads, N * P / 256)
+KERNEL void __launch_bounds__(256) wkv_chunk_carry_kernel(const WkvChunkArgs g)
+{
+    const WkvArgs& a = g.a;
+    const int sp = bid_x(), h = bid_y(), e = bid_z() * 256 + tid();
+    const int N = a.N, P = a.P;
+    if (e >= N * P) return;
+    const int r0 = a.span_row0[sp], chunks = (a.span_rows[sp] + WKC_L - 1) / WKC_L, c0 = g.span_chunk0[sp];
+    float* st = a.state + ((long long)a.row_seq[r0] * a.heads + h) * (long long)N * P;
+    float S = a.row_pos[r0] > 0 ? st[e] : 0.0f;
+    for (int c = c0; c < c0 + chunks; c++)
+    {
+        float* z = g.zbuf + ((long long)c * a.heads + h) * N * P;
+        const float own = z[e];
+        z[e] = S;
+        S = fmaf(g.dbuf[((long long)c * a.heads + h) * N + e / P], S, own);
+    }
+    st[e] = S;
+}
+
+// grid (chunks, heads)
+template <typename T>
+KERNEL void __launch_bounds__(256) wkv_chunk_out_kernel(const WkvChunkArgs g)
+{
+    DYN_SMEM(smem);
+    const WkvArgs& a = g.a;
+    const int c = bid_x(), h = bid_y(), N = a.N, P = a.P, NS = N + 1, LS = WKC_L + 1;
+    int sp, r0, n;
+    wkc_locate(g, c, sp, r0, n);
+    float* cc = (float*)smem;                                    // [L + 1][NS]
+    float* sr = cc + (WKC_L + 1) * NS;                           // [L][NS]
+    float* sk = sr + WKC_L * NS;                                 // [L][NS]
+    float* sv = sk + WKC_L * NS;                                 // [L][P]
+    float* sS = sv + WKC_L * P;                                  // [N][P]
+    float* sA = sS + N * P;                                      // [L][LS]
+    float* so = sA + WKC_L * LS;                                 // [L][P]
+    float* su = so + WKC_L * P;                                  // [N]
+    wkc_log_decay_sums(a, h, r0, n, cc, NS);
+    for (int i = tid(); i < n * N; i += 256)
+    {
+        const int t = i / N, ch = i % N;
+        const long long at = (long long)(r0 + t) * a.ld + h * N + ch;
+        sr[t * NS + ch] = a.r[at];
+        sk[t * NS + ch] = a.k[at];
+    }
+    for (int i = tid(); i < n * P; i += 256) sv[i] = a.v[(long long)(r0 + i / P) * a.ld + h * P + i % P];
+    const float* z = g.zbuf + ((long long)c * a.heads + h) * N * P;
+    for (int e = tid(); e < N * P; e += 256) sS[e] = z[e];
+    for (int ch = tid(); ch < N; ch += 256) su[ch] = a.u[h * N + ch];
+    block_sync();
+    // A[t][s]: consecutive threads take consecutive s (rows of sk / cc NS apart: distinct banks), one t per run of WKC_L threads
+    for (int e = tid(); e < n * WKC_L; e += 256)
+    {
+        const int t = e / WKC_L, s2 = e % WKC_L;
+        float acc = 0.0f;
+        if (s2 < t)
+            for (int ch = 0; ch < N; ch++)
+                acc = fmaf(sr[t * NS + ch] * sk[s2 * NS + ch], expf(cc[t * NS + ch] - cc[(s2 + 1) * NS + ch]), acc);
+        else if (s2 == t)
+            for (int ch = 0; ch < N; ch++) acc = fmaf(sr[t * NS + ch] * su[ch], sk[t * NS + ch], acc);
+        sA[t * LS + s2] = acc;
+    }
+    block_sync();
+    for (int i = tid(); i < n * N; i += 256)
+    {
+        const int t = i / N, ch = i % N;
+        sr[t * NS + ch] *= expf(cc[t * NS + ch]);
+    }
+    block_sync();
+    for (int e = tid(); e < n * P; e += 256)
+    {
+        const int t = e / P, j = e % P;
+        float acc = 0.0f;
+        for (int ch = 0; ch < N; ch++) acc = fmaf(sr[t * NS + ch], sS[ch * P + j], acc);
+        for (int s2 = 0; s2 <= t; s2++) acc = fmaf(sA[t * LS + s2], sv[s2 * P + j], acc);
+        so[e] = acc;
+    }
+    block_sync();
+    for (int t = wave_id(); t < n; t += 4)
+    {
+        float ss = 0.0f;
+        for (int j = lane_id(); j < P; j += 64) { const float ov = so[t * P + j]; ss = fmaf(ov, ov, ss); }
+        ss = wave_allreduce_add(ss);
+        const float rinv = 1.0f / sqrtf(ss / (float)P + a.eps);
+        const long long row = r0 + t;
+        for (int j = lane_id(); j < P; j += 64)
+        {
+            const float gv = a.g[row * a.ld + h * P + j];
+            wk_st<T>((T*)a.out + row * a.ldo + h * P + j, so[t * P + j] * rinv * a.norm_w[h * P + j] * (gv / (1.0f + expf(-gv))));
+        }
+    }
+}
+
+static size_t wkc_out_smem(int N, int P)
+{
+    return sizeof(float) * ((size_t)(WKC_L + 1) * (N + 1) + 2 * (size_t)WKC_L * (N + 1) + 2 * (size_t)WKC_L * P + (size_t)N * P
+                            + (size_t)WKC_L * (WKC_L + 1) + N);
+}
+
 // ---- C ABI ----------------------------------------------------------------------------------------------------------------------
 
 extern "C" int exl2_wkv_mix(const float* h, float* prev, const void* mu, int n_mix, void* out, long long out_stride, const int* row_seq,
@@ -220,6 +397,45 @@ extern "C" int exl2_wkv_scan(const float* r, const float* k, const float* v, con
     const dim3 grid(heads, spans), block((n_val * ks + 63) / 64 * 64);
     if (out_f32) wkv_scan_launch<float>(a, npt, grid, block, smem, stream);
     else wkv_scan_launch<u16>(a, npt, grid, block, smem, stream);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+/* 1 if exl2_wkv_scan_chunked takes this state shape (its staging buffers fit the LDS) */
+extern "C" int exl2_wkv_scan_chunked_supported(int n_key, int n_val)
+{
+    return n_key > 0 && n_val > 0 && wkc_out_smem(n_key, n_val) <= 150 * 1024;
+}
+
+extern "C" int exl2_wkv_scan_chunked(const float* r, const float* k, const float* v, const float* g, int ld, const float* dlog, int ldd,
+                                     const float* u, const float* norm_w, void* out, int ldo, int out_f32, float* state,
+                                     const int* span_row0, const int* span_rows, const int* span_chunk0, int spans, int chunk,
+                                     int total_chunks, const int* row_seq, const int* row_pos, float* zbuf, float* dbuf,
+                                     int heads, int n_key, int n_val, float eps, void* stream)
+{
+    EXL2_REQUIRE(r && k && v && g && dlog && u && norm_w && out && state && span_row0 && span_rows && span_chunk0 && row_seq && row_pos
+                 && zbuf && dbuf, "wkv_scan_chunked: null operand");
+    EXL2_REQUIRE(chunk == WKC_L, "wkv_scan_chunked: chunks are %d rows", WKC_L);
+    EXL2_REQUIRE(heads > 0 && exl2_wkv_scan_chunked_supported(n_key, n_val), "wkv_scan_chunked: state %d x %d does not fit", n_key, n_val);
+    if (spans <= 0 || total_chunks <= 0) return EXL2_OK;
+    WkvChunkArgs c;
+    WkvArgs& a = c.a;
+    a.r = r; a.k = k; a.v = v; a.g = g; a.ld = ld; a.dlog = dlog; a.ldd = ldd; a.u = u; a.norm_w = norm_w; a.out = out; a.ldo = ldo;
+    a.state = state; a.span_row0 = span_row0; a.span_rows = span_rows; a.row_seq = row_seq; a.row_pos = row_pos;
+    a.heads = heads; a.N = n_key; a.P = n_val; a.KS = 1; a.eps = eps;
+    c.span_chunk0 = span_chunk0; c.spans = spans; c.zbuf = zbuf; c.dbuf = dbuf;
+    static bool attr_done[EXL2_MAX_DEVICES];
+    if (exl2_first_on_device(attr_done))
+    {
+        (void)hipFuncSetAttribute((const void*)wkv_chunk_state_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)wkv_chunk_out_kernel<u16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)wkv_chunk_out_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    }
+    const size_t sm1 = sizeof(float) * ((size_t)(2 * WKC_L + 1) * (n_key + 1) + (size_t)WKC_L * n_val);
+    LAUNCH(wkv_chunk_state_kernel, dim3(total_chunks, heads), dim3(256), sm1, stream, c);
+    LAUNCH(wkv_chunk_carry_kernel, dim3(spans, heads, (n_key * n_val + 255) / 256), dim3(256), 0, stream, c);
+    if (out_f32) LAUNCH(wkv_chunk_out_kernel<float>, dim3(total_chunks, heads), dim3(256), wkc_out_smem(n_key, n_val), stream, c);
+    else LAUNCH(wkv_chunk_out_kernel<u16>, dim3(total_chunks, heads), dim3(256), wkc_out_smem(n_key, n_val), stream, c);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;
 }

@@ -1046,6 +1046,26 @@ class ExtC:
                                               self._ptr(row_pos, torch.int32, "row_pos"), int(heads), int(n_key), int(n_val), float(eps),
                                               self._stream(out)))
 
+    def wkv_scan_chunked_supported(self, n_key: int, n_val: int) -> bool:
+        return bool(self.lib.exl2_wkv_scan_chunked_supported(int(n_key), int(n_val)))
+
+    def wkv_scan_chunked(self, rkvg, rows: int, dlog, u, norm_w, out, state, spans, chunks, row_seq, row_pos, zbuf, dbuf, heads: int,
+                         n_key: int, n_val: int, eps: float) -> None:
+        """wkv_scan in chunks; chunks = (span_chunk0 int32 [n], chunk size, chunks in all): zbuf / dbuf hold one entry per chunk"""
+        row0, nrows, n, _longest = spans
+        chunk0, chunk, total = chunks
+        if zbuf.numel() < total * heads * n_key * n_val or dbuf.numel() < total * heads * n_key:
+            raise RuntimeError("wkv_scan_chunked: scratch smaller than the step's chunks")
+        p = self._ptr(rkvg, torch.float32, "rkvg")
+        step = int(rows) * heads * n_key * 4
+        self.lib.check(self.lib.exl2_wkv_scan_chunked(
+            p, p + step, p + 2 * step, p + 3 * step, heads * n_key, self._ptr(dlog, torch.float32, "dlog"), dlog.shape[-1],
+            self._ptr(u, torch.float32, "u"), self._ptr(norm_w, torch.float32, "norm_w"), self._ptr(out, None, "out"), out.shape[-1],
+            int(out.dtype is torch.float32), self._ptr(state, torch.float32, "state"), self._ptr(row0, torch.int32, "span_row0"),
+            self._ptr(nrows, torch.int32, "span_rows"), self._ptr(chunk0, torch.int32, "span_chunk0"), int(n), int(chunk), int(total),
+            self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"), self._ptr(zbuf, torch.float32, "zbuf"),
+            self._ptr(dbuf, torch.float32, "dbuf"), int(heads), int(n_key), int(n_val), float(eps), self._stream(out)))
+
     def graph_begin_capture(self, stream: int | None) -> None:
         self.lib.check(self.lib.exl2_graph_begin_capture(stream))
 

@@ -20,6 +20,7 @@ from .dense_linear import DenseLinear
 class DecayLinearAttention:
     input_f32 = True                                          # forward() takes the normed layer input as fp32 rows
     MIXES = ("r", "k", "v", "g", "w")
+    CHUNKED_FROM = 8                                          # longest span of a step from which the chunked scan is taken
 
     def __init__(self, model, key: str, layer_idx: int, *, heads: int, dim: int):
         self.model, self.ext, self.key, self.layer_idx = model, model.ext, key, layer_idx
@@ -28,6 +29,7 @@ class DecayLinearAttention:
         if heads <= 0 or dim <= 0:
             raise ValueError(f"{key}: {heads} heads of {dim}")
         self.kv_from = None
+        self.chunked_ok = self.ext.wkv_scan_chunked_supported(dim, dim)
 
     def load(self, get):
         """`get(name)` returns the device tensor `<layer>.mix.<name>` in the model's operand dtype"""
@@ -70,6 +72,15 @@ class DecayLinearAttention:
         t = self.w1.forward(x, rows, out=m.buf("wkv.t", (rows, self.rank), m.dtype), epi=ext.EPI_TANH, x_off=4 * rows * width, ldx=width)
         d = self.w2.forward(t, rows, out=m.buf("wkv.d", (rows, inner), f32), bias=self.w0)
         g = m.buf("wkv.g", (rows, inner), m.dtype)
-        ext.wkv_scan(f, rows, d, self.u, self.norm_w, g, st["S"], batch.spans_dev, batch.row_seq, batch.row_pos, self.heads, self.dim,
-                     self.dim, m.norm_eps)
+        if batch.span_chunks is not None and batch.spans_dev[3] >= self.CHUNKED_FROM and self.chunked_ok:
+            # portions of prompts: the recurrence unrolled in chunks, every (chunk, head) independent work
+            total = batch.span_chunks[2]
+            zbuf = m.buf("wkv.z", (total, self.heads, self.dim, self.dim), f32)
+            dbuf = m.buf("wkv.dk", (total, self.heads, self.dim), f32)
+            ext.wkv_scan_chunked(f, rows, d, self.u, self.norm_w, g, st["S"], batch.spans_dev, batch.span_chunks, batch.row_seq, batch.row_pos,
+                                 zbuf, dbuf, self.heads, self.dim, self.dim, m.norm_eps)
+        else:
+            # decoded tokens and short portions: one pass per (span, head) with the state in registers
+            ext.wkv_scan(f, rows, d, self.u, self.norm_w, g, st["S"], batch.spans_dev, batch.row_seq, batch.row_pos, self.heads, self.dim,
+                         self.dim, m.norm_eps)
         return self.o.forward(g, rows, out=m.buf("mix.y", (rows, width), f32))

@@ -575,6 +575,16 @@ int exl2_wkv_scan(const float* r, const float* k, const float* v, const float* g
                   const float* u, const float* norm_w, void* out, int ldo, int out_f32, float* state,
                   const int* span_row0, const int* span_rows, int spans, const int* row_seq, const int* row_pos,
                   int heads, int n_key, int n_val, float eps, void* stream);
+/* exl2_wkv_scan for portions of prompts: the recurrence unrolled in chunks of `chunk` (64) rows, every (chunk, head) independent
+   work around a short carry over each span's chunks; every exponent is evaluated as a non-positive difference.  span_chunk0[i] =
+   number of chunks of the spans before i; zbuf fp32 [total_chunks, heads, n_key, n_val] and dbuf fp32 [total_chunks, heads, n_key]
+   are scratch.  State shapes for which exl2_wkv_scan_chunked_supported returns 1. */
+int exl2_wkv_scan_chunked_supported(int n_key, int n_val);
+int exl2_wkv_scan_chunked(const float* r, const float* k, const float* v, const float* g, int ld, const float* dlog, int ldd,
+                          const float* u, const float* norm_w, void* out, int ldo, int out_f32, float* state,
+                          const int* span_row0, const int* span_rows, const int* span_chunk0, int spans, int chunk,
+                          int total_chunks, const int* row_seq, const int* row_pos, float* zbuf, float* dbuf,
+                          int heads, int n_key, int n_val, float eps, void* stream);
 
 #ifdef __cplusplus
 }

@@ -293,10 +293,14 @@ def test_blends_with_the_previous_input(be, dtype):
     assert close(be.n(prev)[0], last[0], 0) and close(be.n(prev)[2], last[2], 0)
 
 
+@pytest.mark.parametrize("chunked", [False, True, "alternating"])
 @pytest.mark.parametrize("heads,D", [(3, 8), (2, 64), (1, 5), (4, 32), (2, 100), (1, 128)])
-def test_decaying_state_over_spans_and_steps(be, heads, D):
-    """portions of 1 .. 37 tokens of two sequences: the state carried in the slot gives what one pass over the whole sequence gives;
-    a slot's stale state is not seen by a sequence that starts at position 0"""
+def test_decaying_state_over_spans_and_steps(be, heads, D, chunked):
+    """portions of 1 .. 150 tokens of two sequences: the state carried in the slot gives what one pass over the whole sequence gives;
+    a slot's stale state is not seen by a sequence that starts at position 0.  Token by token, unrolled in chunks (several chunks, chunks
+    that end early, decays fast enough that a factored exponential would overflow), and both forms alternating on the same slots"""
+    if chunked and not be.ext.wkv_scan_chunked_supported(D, D):
+        pytest.skip("the chunked form does not take this state size")
     rng = np.random.default_rng(heads * 100 + D)
     inner, eps = heads * D, 1e-5
     u = ON.bf16_round(rng.standard_normal((heads, D)) * 0.5)
@@ -304,16 +308,24 @@ def test_decaying_state_over_spans_and_steps(be, heads, D):
     state = torch.full((3, heads, D, D), 5.0, dtype=F32, device=be.device)
     S = {1: np.zeros((heads, D, D)), 2: np.zeros((heads, D, D))}
     n_tok = {1: 0, 2: 0}
-    for step in ([(1, 2), (2, 1)], [(2, 37), (1, 1)], [(1, 1)], [(1, 17), (2, 3)], [(2, 1), (1, 1)]):
+    for n_step, step in enumerate(([(1, 2), (2, 1)], [(2, 37), (1, 1)], [(1, 1)], [(1, 150), (2, 3)], [(2, 1), (1, 1)], [(2, 64), (1, 65)])):
         lens = [n for _s, n in step]
         rows = sum(lens)
         f = rng.standard_normal((4, rows, inner)).astype(np.float32)
         f[1] *= 0.5
         dlog = (rng.standard_normal((rows, inner)) - 1.0).astype(np.float32)
+        dlog[:, ::3] += 2.5                                      # channels that forget within a few tokens
         seq = np.concatenate([[s] * n for s, n in step])
         pos = np.concatenate([np.arange(n_tok[s], n_tok[s] + n) for s, n in step])
         out = torch.zeros((rows, inner), dtype=F32, device=be.device)
-        be.ext.wkv_scan(be.t(f), rows, be.t(dlog), be.t(u), be.t(nw), out, state, spans_of(be, lens), ints(be, seq), ints(be, pos), heads, D, D, eps)
+        if chunked is True or (chunked and n_step % 2 == 1):
+            chunk0 = np.cumsum([0] + [-(-n // 64) for n in lens])
+            zbuf = torch.zeros((int(chunk0[-1]), heads, D, D), dtype=F32, device=be.device)
+            dbuf = torch.zeros((int(chunk0[-1]), heads, D), dtype=F32, device=be.device)
+            be.ext.wkv_scan_chunked(be.t(f), rows, be.t(dlog), be.t(u), be.t(nw), out, state, spans_of(be, lens), (ints(be, chunk0[:-1]), 64, int(chunk0[-1])),
+                                    ints(be, seq), ints(be, pos), zbuf, dbuf, heads, D, D, eps)
+        else:
+            be.ext.wkv_scan(be.t(f), rows, be.t(dlog), be.t(u), be.t(nw), out, state, spans_of(be, lens), ints(be, seq), ints(be, pos), heads, D, D, eps)
         got, r = be.n(out), 0
         for s, n in step:
             for _ in range(n):
