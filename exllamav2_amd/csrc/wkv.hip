@@ -206,42 +206,89 @@ DEV void wkc_log_decay_sums(const WkvArgs& a, int h, int r0, int n, float* cc, i
         cc[t * NS + ch] = t == 0 ? 0.0f : -expf(a.dlog[(long long)(r0 + t - 1) * a.ldd + h * N + ch]);
     }
     block_sync();
+    // running sums in two levels: segments of 8 tokens by N x 8 threads, then every channel's thread adds the sum of the segments in
+    // front to the later segments (independent updates: only the 8 segment totals form a chain)
+    for (int i = tid(); i < N * (WKC_L / 8); i += nthreads())
+    {
+        const int ch = i % N, t0 = (i / N) * 8;
+        float run = 0.0f;
+        #pragma unroll
+        for (int q = 1; q <= 8; q++)
+            if (t0 + q <= n) { run += cc[(t0 + q) * NS + ch]; cc[(t0 + q) * NS + ch] = run; }
+    }
+    block_sync();
     for (int ch = tid(); ch < N; ch += nthreads())
     {
+        float off[WKC_L / 8];
         float run = 0.0f;
-        for (int t = 1; t <= n; t++) { run += cc[t * NS + ch]; cc[t * NS + ch] = run; }
+        #pragma unroll
+        for (int sg = 0; sg < WKC_L / 8; sg++)
+        {
+            off[sg] = run;
+            if (sg * 8 < n) run += cc[min(sg * 8 + 8, n) * NS + ch];
+        }
+        #pragma unroll
+        for (int sg = 1; sg < WKC_L / 8; sg++)
+            #pragma unroll
+            for (int q = 1; q <= 8; q++)
+                if (sg * 8 + q <= n) cc[(sg * 8 + q) * NS + ch] += off[sg];
     }
     block_sync();
 }
 
 // grid (chunks, heads)
-KERNEL void __launch_bounds__(256) wkv_chunk_state_kernel(const WkvChunkArgs g)
+KERNEL void __launch_bounds__(512) wkv_chunk_state_kernel(const WkvChunkArgs g)
 {
     DYN_SMEM(smem);
     const WkvArgs& a = g.a;
     const int c = bid_x(), h = bid_y(), N = a.N, P = a.P, NS = N + 1;
     int sp, r0, n;
     wkc_locate(g, c, sp, r0, n);
-    float* cc = (float*)smem;                                    // [L + 1][NS]
+    float* sv = (float*)smem;                                    // [L][P] (first: 16-byte aligned rows when P % 4 == 0)
+    float* cc = sv + WKC_L * P;                                  // [L + 1][NS]
     float* kd = cc + (WKC_L + 1) * NS;                           // [L][NS]
-    float* sv = kd + WKC_L * NS;                                 // [L][P]
     wkc_log_decay_sums(a, h, r0, n, cc, NS);
-    for (int i = tid(); i < n * N; i += 256)
+    for (int i = tid(); i < n * N; i += nthreads())
     {
         const int t = i / N, ch = i % N;
         kd[t * NS + ch] = expf(cc[n * NS + ch] - cc[(t + 1) * NS + ch]) * a.k[(long long)(r0 + t) * a.ld + h * N + ch];
     }
-    for (int i = tid(); i < n * P; i += 256) sv[i] = a.v[(long long)(r0 + i / P) * a.ld + h * P + i % P];
+    for (int i = tid(); i < n * P; i += nthreads()) sv[i] = a.v[(long long)(r0 + i / P) * a.ld + h * P + i % P];
     block_sync();
     float* z = g.zbuf + ((long long)c * a.heads + h) * N * P;
-    for (int e = tid(); e < N * P; e += 256)
+    if (N % 4 == 0 && P % 4 == 0)
     {
-        const int ch = e / P, j = e % P;
-        float acc = 0.0f;
-        for (int t = 0; t < n; t++) acc = fmaf(kd[t * NS + ch], sv[t * P + j], acc);
-        z[e] = acc;
+        // 4 x 4 outputs per thread: every staged value feeds four products
+        for (int e = tid(); e < (N / 4) * (P / 4); e += nthreads())
+        {
+            const int ch = (e / (P / 4)) * 4, j = (e % (P / 4)) * 4;
+            float acc[4][4] = {};
+            #pragma unroll 2
+            for (int t = 0; t < n; t++)
+            {
+                const f32x4 vv = *(const f32x4*)(sv + t * P + j);
+                #pragma unroll
+                for (int q = 0; q < 4; q++)
+                {
+                    const float kq = kd[t * NS + ch + q];
+                    acc[q][0] = fmaf(kq, vv[0], acc[q][0]); acc[q][1] = fmaf(kq, vv[1], acc[q][1]);
+                    acc[q][2] = fmaf(kq, vv[2], acc[q][2]); acc[q][3] = fmaf(kq, vv[3], acc[q][3]);
+                }
+            }
+            #pragma unroll
+            for (int q = 0; q < 4; q++) *(f32x4*)(z + (ch + q) * P + j) = (f32x4){acc[q][0], acc[q][1], acc[q][2], acc[q][3]};
+        }
     }
-    for (int ch = tid(); ch < N; ch += 256) g.dbuf[((long long)c * a.heads + h) * N + ch] = expf(cc[n * NS + ch]);
+    else
+        for (int e = tid(); e < N * P; e += nthreads())
+        {
+            const int ch = e / P, j = e % P;
+            float acc = 0.0f;
+            #pragma unroll 4
+            for (int t = 0; t < n; t++) acc = fmaf(kd[t * NS + ch], sv[t * P + j], acc);
+            z[e] = acc;
+        }
+    for (int ch = tid(); ch < N; ch += nthreads()) g.dbuf[((long long)c * a.heads + h) * N + ch] = expf(cc[n * NS + ch]);
 }
 
 // grid (spans, heads, N * P / 256)
@@ -266,63 +313,91 @@ KERNEL void __launch_bounds__(256) wkv_chunk_carry_kernel(const WkvChunkArgs g)
 
 // grid (chunks, heads)
 template <typename T>
-KERNEL void __launch_bounds__(256) wkv_chunk_out_kernel(const WkvChunkArgs g)
+KERNEL void __launch_bounds__(1024) wkv_chunk_out_kernel(const WkvChunkArgs g)
 {
     DYN_SMEM(smem);
     const WkvArgs& a = g.a;
     const int c = bid_x(), h = bid_y(), N = a.N, P = a.P, NS = N + 1, LS = WKC_L + 1;
     int sp, r0, n;
     wkc_locate(g, c, sp, r0, n);
-    float* cc = (float*)smem;                                    // [L + 1][NS]
-    float* sr = cc + (WKC_L + 1) * NS;                           // [L][NS]
-    float* sk = sr + WKC_L * NS;                                 // [L][NS]
-    float* sv = sk + WKC_L * NS;                                 // [L][P]
-    float* sS = sv + WKC_L * P;                                  // [N][P]
-    float* sA = sS + N * P;                                      // [L][LS]
-    float* so = sA + WKC_L * LS;                                 // [L][P]
-    float* su = so + WKC_L * P;                                  // [N]
+    // four regions, two of them used twice (so that two workgroups share a CU's LDS at 64 x 64): the decay sums give way to the
+    // values, the keys to the outputs; the state entering the chunk is read from memory where it is used
+    const int PS = max(NS, P);
+    float* cc = (float*)smem;                                    // [L + 1][PS]: decay sums (rows of NS), later the values [L][P]
+    float* sr = cc + (WKC_L + 1) * PS;                           // [L][NS]
+    float* sk = sr + WKC_L * NS;                                 // [L][PS]: keys (rows of NS), later the outputs [L][P]
+    float* sA = sk + WKC_L * PS;                                 // [L][LS]
+    float* su = sA + WKC_L * LS;                                 // [N]
+    float* sv = cc; float* so = sk;
+    const float* sS = g.zbuf + ((long long)c * a.heads + h) * N * P;
     wkc_log_decay_sums(a, h, r0, n, cc, NS);
-    for (int i = tid(); i < n * N; i += 256)
+    for (int i = tid(); i < n * N; i += nthreads())
     {
         const int t = i / N, ch = i % N;
         const long long at = (long long)(r0 + t) * a.ld + h * N + ch;
         sr[t * NS + ch] = a.r[at];
         sk[t * NS + ch] = a.k[at];
     }
-    for (int i = tid(); i < n * P; i += 256) sv[i] = a.v[(long long)(r0 + i / P) * a.ld + h * P + i % P];
-    const float* z = g.zbuf + ((long long)c * a.heads + h) * N * P;
-    for (int e = tid(); e < N * P; e += 256) sS[e] = z[e];
-    for (int ch = tid(); ch < N; ch += 256) su[ch] = a.u[h * N + ch];
+    for (int ch = tid(); ch < N; ch += nthreads()) su[ch] = a.u[h * N + ch];
     block_sync();
-    // A[t][s]: consecutive threads take consecutive s (rows of sk / cc NS apart: distinct banks), one t per run of WKC_L threads
-    for (int e = tid(); e < n * WKC_L; e += 256)
+    // A[t][s], s < t: a run of WKC_L threads takes rows t and WKC_L - 1 - t together (t + (WKC_L - 1 - t) entries below the diagonal:
+    // every lane has work); consecutive threads take consecutive s (rows of sk / cc NS apart: distinct banks).  The diagonal and the
+    // zeros above it come first.
+    for (int e = tid(); e < WKC_L * WKC_L; e += nthreads())
     {
         const int t = e / WKC_L, s2 = e % WKC_L;
         float acc = 0.0f;
-        if (s2 < t)
-            for (int ch = 0; ch < N; ch++)
-                acc = fmaf(sr[t * NS + ch] * sk[s2 * NS + ch], expf(cc[t * NS + ch] - cc[(s2 + 1) * NS + ch]), acc);
-        else if (s2 == t)
+        if (s2 == t && t < n)
             for (int ch = 0; ch < N; ch++) acc = fmaf(sr[t * NS + ch] * su[ch], sk[t * NS + ch], acc);
+        if (s2 >= t) sA[t * LS + s2] = acc;
+    }
+    for (int e = tid(); e < (WKC_L / 2) * WKC_L; e += nthreads())
+    {
+        const int pair = e / WKC_L, l = e % WKC_L;
+        const int t = l < pair ? pair : WKC_L - 1 - pair, s2 = l < pair ? l : l - pair;
+        if (s2 >= t || t >= n) continue;
+        const float* rt = sr + t * NS; const float* ct = cc + t * NS;
+        const float* ks = sk + s2 * NS; const float* cs = cc + (s2 + 1) * NS;
+        float acc = 0.0f;
+        #pragma unroll 8
+        for (int ch = 0; ch < N; ch++) acc = fmaf(rt[ch] * ks[ch], fast_exp(ct[ch] - cs[ch]), acc);
         sA[t * LS + s2] = acc;
     }
     block_sync();
-    for (int i = tid(); i < n * N; i += 256)
+    for (int i = tid(); i < n * N; i += nthreads())
     {
         const int t = i / N, ch = i % N;
         sr[t * NS + ch] *= expf(cc[t * NS + ch]);
     }
+    block_sync();                                                // the decay sums and the keys have been used: their regions take v and o
+    for (int i = tid(); i < n * P; i += nthreads()) sv[i] = a.v[(long long)(r0 + i / P) * a.ld + h * P + i % P];
     block_sync();
-    for (int e = tid(); e < n * P; e += 256)
+    // four rows of the chunk per thread share every read of the state and of a value row (A is zero above the diagonal)
+    for (int e = tid(); e < (WKC_L / 4) * P; e += nthreads())
     {
-        const int t = e / P, j = e % P;
-        float acc = 0.0f;
-        for (int ch = 0; ch < N; ch++) acc = fmaf(sr[t * NS + ch], sS[ch * P + j], acc);
-        for (int s2 = 0; s2 <= t; s2++) acc = fmaf(sA[t * LS + s2], sv[s2 * P + j], acc);
-        so[e] = acc;
+        const int t0 = (e / P) * 4, j = e % P;
+        if (t0 >= n) continue;
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        #pragma unroll 4
+        for (int ch = 0; ch < N; ch++)
+        {
+            const float sv2 = sS[ch * P + j];
+            #pragma unroll
+            for (int q = 0; q < 4; q++) acc[q] = fmaf(sr[(t0 + q) * NS + ch], sv2, acc[q]);
+        }
+        const int s_hi = min(t0 + 3, n - 1);
+        #pragma unroll 4
+        for (int s2 = 0; s2 <= s_hi; s2++)
+        {
+            const float vv = sv[s2 * P + j];
+            #pragma unroll
+            for (int q = 0; q < 4; q++) acc[q] = fmaf(sA[(t0 + q) * LS + s2], vv, acc[q]);
+        }
+        #pragma unroll
+        for (int q = 0; q < 4; q++) if (t0 + q < n) so[(t0 + q) * P + j] = acc[q];
     }
     block_sync();
-    for (int t = wave_id(); t < n; t += 4)
+    for (int t = wave_id(); t < n; t += nthreads() / 64)
     {
         float ss = 0.0f;
         for (int j = lane_id(); j < P; j += 64) { const float ov = so[t * P + j]; ss = fmaf(ov, ov, ss); }
@@ -339,8 +414,8 @@ KERNEL void __launch_bounds__(256) wkv_chunk_out_kernel(const WkvChunkArgs g)
 
 static size_t wkc_out_smem(int N, int P)
 {
-    return sizeof(float) * ((size_t)(WKC_L + 1) * (N + 1) + 2 * (size_t)WKC_L * (N + 1) + 2 * (size_t)WKC_L * P + (size_t)N * P
-                            + (size_t)WKC_L * (WKC_L + 1) + N);
+    const size_t ps = N + 1 > P ? N + 1 : P;
+    return sizeof(float) * ((size_t)(2 * WKC_L + 1) * ps + (size_t)WKC_L * (N + 1) + (size_t)WKC_L * (WKC_L + 1) + N);
 }
 
 // ---- C ABI ----------------------------------------------------------------------------------------------------------------------
@@ -432,10 +507,10 @@ extern "C" int exl2_wkv_scan_chunked(const float* r, const float* k, const float
         (void)hipFuncSetAttribute((const void*)wkv_chunk_out_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     }
     const size_t sm1 = sizeof(float) * ((size_t)(2 * WKC_L + 1) * (n_key + 1) + (size_t)WKC_L * n_val);
-    LAUNCH(wkv_chunk_state_kernel, dim3(total_chunks, heads), dim3(256), sm1, stream, c);
+    LAUNCH(wkv_chunk_state_kernel, dim3(total_chunks, heads), dim3(512), sm1, stream, c);
     LAUNCH(wkv_chunk_carry_kernel, dim3(spans, heads, (n_key * n_val + 255) / 256), dim3(256), 0, stream, c);
-    if (out_f32) LAUNCH(wkv_chunk_out_kernel<float>, dim3(total_chunks, heads), dim3(256), wkc_out_smem(n_key, n_val), stream, c);
-    else LAUNCH(wkv_chunk_out_kernel<u16>, dim3(total_chunks, heads), dim3(256), wkc_out_smem(n_key, n_val), stream, c);
+    if (out_f32) LAUNCH(wkv_chunk_out_kernel<float>, dim3(total_chunks, heads), dim3(1024), wkc_out_smem(n_key, n_val), stream, c);
+    else LAUNCH(wkv_chunk_out_kernel<u16>, dim3(total_chunks, heads), dim3(1024), wkc_out_smem(n_key, n_val), stream, c);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;
 }
