@@ -346,10 +346,15 @@ KERNEL void __launch_bounds__(1024) wkv_chunk_out_kernel(const WkvChunkArgs g)
     for (int e = tid(); e < WKC_L * WKC_L; e += nthreads())
     {
         const int t = e / WKC_L, s2 = e % WKC_L;
+        if (s2 > t) sA[t * LS + s2] = 0.0f;
+    }
+    for (int t = tid(); t < WKC_L; t += nthreads())              // the diagonal: one thread per row, the rows side by side in a wave
+    {
         float acc = 0.0f;
-        if (s2 == t && t < n)
+        if (t < n)
+            #pragma unroll 8
             for (int ch = 0; ch < N; ch++) acc = fmaf(sr[t * NS + ch] * su[ch], sk[t * NS + ch], acc);
-        if (s2 >= t) sA[t * LS + s2] = acc;
+        sA[t * LS + t] = acc;
     }
     for (int e = tid(); e < (WKC_L / 2) * WKC_L; e += nthreads())
     {
