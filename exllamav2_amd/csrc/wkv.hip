@@ -58,7 +58,7 @@ KERNEL void __launch_bounds__(256) wkv_mix_kernel(const MixArgs a)
 // ---- the recurrence, token by token ---------------------------------------------------------------------------------------------------
 
 #define WKV_CHUNK 16                         // tokens staged in LDS per round
-#define WKV_MAX_NPT 128                      // state rows per thread
+#define WKV_MAX_NPT 256                      // state rows per thread
 
 struct WkvArgs
 {
@@ -94,15 +94,16 @@ KERNEL void __launch_bounds__(256) wkv_scan_kernel(const WkvArgs a)
     float* s_v = s_w + WKV_CHUNK * N;                            // [CHUNK, P]
     float* s_o = s_v + WKV_CHUNK * P;                            // [CHUNK, P]
     float* s_part = s_o + WKV_CHUNK * P;                         // [CHUNK, KS, P]
+    float* s_u = s_part + WKV_CHUNK * KS * P;                    // [N]
     float* st = a.state + ((long long)a.row_seq[r0] * a.heads + h) * (long long)N * P;
-    float S[NPT], U[NPT];
+    float S[NPT];
     #pragma unroll
     for (int i = 0; i < NPT; i++)
     {
         const int n = j + KS * i;
         S[i] = (owner && pos0 > 0 && n < N) ? st[(long long)n * P + p] : 0.0f;
-        U[i] = n < N ? a.u[h * N + n] : 0.0f;
     }
+    for (int i = t; i < N; i += nt) s_u[i] = a.u[h * N + i];
     for (int c0 = 0; c0 < n_tok; c0 += WKV_CHUNK)
     {
         const int nc = min(WKV_CHUNK, n_tok - c0);
@@ -128,7 +129,7 @@ KERNEL void __launch_bounds__(256) wkv_scan_kernel(const WkvArgs a)
                 if (n < N)
                 {
                     const float kv = s_k[kk * N + n] * vv;
-                    part = fmaf(s_r[kk * N + n], fmaf(U[i], kv, S[i]), part);
+                    part = fmaf(s_r[kk * N + n], fmaf(s_u[n], kv, S[i]), part);
                     S[i] = fmaf(s_w[kk * N + n], S[i], kv);
                 }
             }
@@ -451,6 +452,7 @@ static void wkv_scan_launch(const WkvArgs& a, int npt, dim3 grid, dim3 block, si
     else if (npt <= 16) LAUNCH((wkv_scan_kernel<T, 16>), grid, block, smem, stream, a);
     else if (npt <= 32) LAUNCH((wkv_scan_kernel<T, 32>), grid, block, smem, stream, a);
     else if (npt <= 64) LAUNCH((wkv_scan_kernel<T, 64>), grid, block, smem, stream, a);
+    else if (npt <= 128) LAUNCH((wkv_scan_kernel<T, 128>), grid, block, smem, stream, a);
     else LAUNCH((wkv_scan_kernel<T, WKV_MAX_NPT>), grid, block, smem, stream, a);
 }
 
@@ -472,8 +474,21 @@ extern "C" int exl2_wkv_scan(const float* r, const float* k, const float* v, con
     a.r = r; a.k = k; a.v = v; a.g = g; a.ld = ld; a.dlog = dlog; a.ldd = ldd; a.u = u; a.norm_w = norm_w; a.out = out; a.ldo = ldo;
     a.state = state; a.span_row0 = span_row0; a.span_rows = span_rows; a.row_seq = row_seq; a.row_pos = row_pos;
     a.heads = heads; a.N = n_key; a.P = n_val; a.KS = ks; a.eps = eps;
-    const size_t smem = sizeof(float) * ((size_t)WKV_CHUNK * (3 * n_key + 2 * n_val + (size_t)ks * n_val));
-    EXL2_REQUIRE(smem <= 64 * 1024, "wkv_scan: state %d x %d does not fit the staging buffers", n_key, n_val);
+    const size_t smem = sizeof(float) * ((size_t)WKV_CHUNK * (3 * n_key + 2 * n_val + (size_t)ks * n_val) + n_key);
+    EXL2_REQUIRE(smem <= 150 * 1024, "wkv_scan: state %d x %d does not fit the staging buffers", n_key, n_val);
+    if (smem > 48 * 1024)
+    {
+        static bool attr_done[EXL2_MAX_DEVICES];
+        if (exl2_first_on_device(attr_done))
+        {
+            (void)hipFuncSetAttribute((const void*)wkv_scan_kernel<u16, 128>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)wkv_scan_kernel<float, 128>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)wkv_scan_kernel<u16, WKV_MAX_NPT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)wkv_scan_kernel<float, WKV_MAX_NPT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)wkv_scan_kernel<u16, 64>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)wkv_scan_kernel<float, 64>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        }
+    }
     const dim3 grid(heads, spans), block((n_val * ks + 63) / 64 * 64);
     if (out_f32) wkv_scan_launch<float>(a, npt, grid, block, smem, stream);
     else wkv_scan_launch<u16>(a, npt, grid, block, smem, stream);

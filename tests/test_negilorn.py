@@ -294,7 +294,7 @@ def test_blends_with_the_previous_input(be, dtype):
 
 
 @pytest.mark.parametrize("chunked", [False, True, "alternating"])
-@pytest.mark.parametrize("heads,D", [(3, 8), (2, 64), (1, 5), (4, 32), (2, 100), (1, 128)])
+@pytest.mark.parametrize("heads,D", [(3, 8), (2, 64), (1, 5), (4, 32), (2, 100), (1, 128), (1, 192)])
 def test_decaying_state_over_spans_and_steps(be, heads, D, chunked):
     """portions of 1 .. 150 tokens of two sequences: the state carried in the slot gives what one pass over the whole sequence gives;
     a slot's stale state is not seen by a sequence that starts at position 0.  Token by token, unrolled in chunks (several chunks, chunks
