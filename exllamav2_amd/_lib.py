@@ -134,7 +134,7 @@ PROTOTYPES = {
     # scalar-gain RMS norm + token shift, sigmoid router (csrc/rowops.hip); decaying linear attention (csrc/wkv.hip)
     "exl2_add_rms_shift": (ci, [vp, vp, vp, ci, cf, cf, vp, vp, vp, vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]),
     "exl2_span_last_rows": (ci, [vp, ci, vp, ci, vp, vp, ci, vp, vp]),
-    "exl2_moe_route_sigmoid": (ci, [vp, vp, vp, ci, ci, ci, cf, vp, vp, vp, vp]),
+    "exl2_moe_route_sigmoid": (ci, [vp, vp, vp, ci, ci, ci, cf, ci, vp, vp, vp, vp]),
     "exl2_wkv_mix": (ci, [vp, vp, vp, ci, vp, cll, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]),
     "exl2_wkv_scan": (ci, [vp, vp, vp, vp, ci, vp, ci, vp, vp, vp, ci, ci, vp, vp, vp, ci, vp, vp, ci, ci, ci, cf, vp]),
     "exl2_wkv_scan_chunked_supported": (ci, [ci, ci]),

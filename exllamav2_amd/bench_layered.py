@@ -297,7 +297,7 @@ def shift_config(s: dict) -> dict:
             layers.append({"type": "wkv", "mlp": None, "mixer": {"dim": s["wkv_dim"], "heads": s["wkv_heads"]}})
         else:
             m = {"dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv_heads"], "vdim": s["vdim"], "mask": {"size": s["chunk"]},
-                 "scale": s["dim"] ** -0.5, "softcap": 50.0,
+                 "scale": s["dim"] ** -0.5, "softcap": 30.0,
                  "rot": {"base": 500000.0, "dims": s["rot_dims"], "scaling": {"factor": 8.0, "original": 8192, "low": 1.0, "high": 4.0}}}
             if ch == "k":
                 m["kv_from"] = last_attn

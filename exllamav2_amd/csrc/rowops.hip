@@ -320,12 +320,13 @@ KERNEL void __launch_bounds__(256) span_last_row_kernel(const float* src, int ld
 // ---- router -----------------------------------------------------------------------------------------------------------------
 // One wave per token.  logits fp32 [rows, n_total]; scores = softmax over all n_total; the `top` largest (score + correction) win
 // (first index on a tie); weight = score / (sum of the chosen scores + 1e-20) * scale.  sigmoid_scores: scores = sigmoid(logits),
-// each on its own, and the weights are the chosen scores times scale (no renormalisation).
+// each on its own, and the weights are the chosen scores times scale (no renormalisation).  Rows of ids / wts are `ld` values apart;
+// extra_id >= 0: column `top` of every row names that expert with weight 1 (an expert every token uses, run with the chosen ones).
 
 #define ROUTE_MAX_PER_LANE 8
 
 KERNEL void __launch_bounds__(64) moe_route_kernel(const float* logits, const float* correction, int* ids, float* wts,
-                                                    int n_total, int top, float scale, int sigmoid_scores)
+                                                    int n_total, int top, float scale, int sigmoid_scores, int ld, int extra_id)
 {
     const int r = bid_x();
     const int lane = lane_id();
@@ -382,9 +383,10 @@ KERNEL void __launch_bounds__(64) moe_route_kernel(const float* logits, const fl
     }
     if (lane < top)
     {
-        ids[r * top + lane] = my_id;
-        wts[r * top + lane] = sigmoid_scores ? my_w * scale : my_w / (chosen_sum + 1e-20f) * scale;
+        ids[r * ld + lane] = my_id;
+        wts[r * ld + lane] = sigmoid_scores ? my_w * scale : my_w / (chosen_sum + 1e-20f) * scale;
     }
+    if (extra_id >= 0 && lane == 0) { ids[r * ld + top] = extra_id; wts[r * ld + top] = 1.0f; }
 }
 
 // per-expert row lists for the grouped linear, in pair order.  Two launches of one workgroup per expert: counts (256 threads, ballot +
@@ -514,36 +516,41 @@ extern "C" int exl2_add_layer_norm(float* x, const float* y, const void* w, cons
 }
 
 static int moe_route_any(const float* logits, const float* correction, int* ids, float* wts, int rows, int n_total, int top,
-                         float scale, int n_real, int* grp_count, int* grp_offset, int* grp_rows, int sigmoid_scores, void* stream);
+                         float scale, int n_real, int* grp_count, int* grp_offset, int* grp_rows, int sigmoid_scores, int shared_slot,
+                         void* stream);
 
 extern "C" int exl2_moe_route_scored(const float* logits, const float* correction, int* ids, float* wts, int rows, int n_total, int top,
                                      float scale, int n_real, int* grp_count, int* grp_offset, int* grp_rows, void* stream)
 {
-    return moe_route_any(logits, correction, ids, wts, rows, n_total, top, scale, n_real, grp_count, grp_offset, grp_rows, 0, stream);
+    return moe_route_any(logits, correction, ids, wts, rows, n_total, top, scale, n_real, grp_count, grp_offset, grp_rows, 0, 0, stream);
 }
 
 extern "C" int exl2_moe_route_sigmoid(const float* logits, int* ids, float* wts, int rows, int n_total, int top, float scale,
-                                      int* grp_count, int* grp_offset, int* grp_rows, void* stream)
+                                      int shared_slot, int* grp_count, int* grp_offset, int* grp_rows, void* stream)
 {
-    return moe_route_any(logits, nullptr, ids, wts, rows, n_total, top, scale, n_total, grp_count, grp_offset, grp_rows, 1, stream);
+    return moe_route_any(logits, nullptr, ids, wts, rows, n_total, top, scale, n_total + (shared_slot ? 1 : 0), grp_count, grp_offset,
+                         grp_rows, 1, shared_slot, stream);
 }
 
 static int moe_route_any(const float* logits, const float* correction, int* ids, float* wts, int rows, int n_total, int top,
-                         float scale, int n_real, int* grp_count, int* grp_offset, int* grp_rows, int sigmoid_scores, void* stream)
+                         float scale, int n_real, int* grp_count, int* grp_offset, int* grp_rows, int sigmoid_scores, int shared_slot,
+                         void* stream)
 {
+    const int ld = top + (shared_slot ? 1 : 0);                  // values per row of ids / wts
     EXL2_REQUIRE(logits && ids && wts, "moe_route_scored: null operand");
     EXL2_REQUIRE(n_total > 0 && n_total <= 64 * ROUTE_MAX_PER_LANE, "moe_route_scored: %d experts (at most %d)", n_total, 64 * ROUTE_MAX_PER_LANE);
     EXL2_REQUIRE(top > 0 && top <= 64 && top <= n_total, "moe_route_scored: top %d of %d", top, n_total);
-    EXL2_REQUIRE(n_real >= 0 && n_real <= n_total, "moe_route_scored: %d experts with weights of %d", n_real, n_total);
+    EXL2_REQUIRE(n_real >= 0 && n_real <= n_total + (shared_slot ? 1 : 0), "moe_route_scored: %d experts with weights of %d", n_real, n_total);
     if (rows <= 0) return EXL2_OK;
-    LAUNCH(moe_route_kernel, dim3(rows), dim3(64), 0, stream, logits, correction, ids, wts, n_total, top, scale, sigmoid_scores);
+    LAUNCH(moe_route_kernel, dim3(rows), dim3(64), 0, stream, logits, correction, ids, wts, n_total, top, scale, sigmoid_scores, ld,
+           shared_slot ? n_total : -1);
     if (grp_count)
     {
         EXL2_REQUIRE(grp_offset && grp_rows, "moe_route_scored: grouped lists need offsets and rows");
         if (n_real > 0)
         {
-            LAUNCH(moe_count_kernel, dim3(n_real), dim3(256), 0, stream, (const int*)ids, rows * top, grp_count);
-            LAUNCH(moe_fill_kernel, dim3(n_real), dim3(64), 0, stream, (const int*)ids, rows * top, (const int*)grp_count, grp_offset, grp_rows);
+            LAUNCH(moe_count_kernel, dim3(n_real), dim3(256), 0, stream, (const int*)ids, rows * ld, grp_count);
+            LAUNCH(moe_fill_kernel, dim3(n_real), dim3(64), 0, stream, (const int*)ids, rows * ld, (const int*)grp_count, grp_offset, grp_rows);
         }
     }
     HIP_TRY(hipGetLastError());

@@ -82,7 +82,8 @@ class Engine:
             dev = self.model.device
             packed = torch.tensor([ids, seq, pos], dtype=torch.int32).to(dev)
             lr = torch.tensor(want_rows or [0], dtype=torch.int32).to(dev)
-            batch = StepBatch(packed[0], packed[1], packed[2], self.pool.device_table(), lr, len(ids), len(want_rows), spans=spans)
+            batch = StepBatch(packed[0], packed[1], packed[2], self.pool.device_table(), lr, len(ids), len(want_rows), spans=spans,
+                              logits_all_rows=want_rows == list(range(len(ids))))
             chunk0, total = [], 0
             for s in spans:                                       # recurrent mixers unroll long spans in chunks of SPAN_CHUNK rows
                 chunk0.append(total)
@@ -121,7 +122,7 @@ class Engine:
             st = {"inputs": torch.zeros((3, b), dtype=torch.int32, device=dev), "rows": ar, "graph": None, "runs": 0}
             cap = self.pool.num_pages * self.pool.page_size
             st["batch"] = StepBatch(st["inputs"][0], st["inputs"][1], st["inputs"][2], self.pool.device_table(), ar, b, b,
-                                    tiles1=(ar, b, cap - 1), spans_dev=(ar, torch.ones_like(ar), b, 1))
+                                    tiles1=(ar, b, cap - 1), spans_dev=(ar, torch.ones_like(ar), b, 1), logits_all_rows=True)
             self._decode[b] = st
         if st["graph"] is not None and st.get("epoch") != getattr(m, "scratch_epoch", 0):
             # a larger step has moved a scratch buffer since the capture: the graph holds the old addresses

@@ -1016,11 +1016,15 @@ class ExtC:
             self._ptr(row0, torch.int32, "span_row0"), self._ptr(nrows, torch.int32, "span_rows"), int(n), int(longest),
             self._dense_code(dt), int(rows), int(width), self._stream(x32)))
 
-    def moe_route_sigmoid(self, logits, ids, wts, rows: int, n_total: int, top: int, scale: float = 1.0, groups=None) -> None:
+    def moe_route_sigmoid(self, logits, ids, wts, rows: int, n_total: int, top: int, scale: float = 1.0, groups=None,
+                          shared_slot: bool = False) -> None:
+        """shared_slot: ids / wts are [rows, top + 1], the last column names expert n_total with weight 1"""
         gc, go, gr = groups if groups is not None else (None, None, None)
+        if ids.numel() < rows * (top + int(shared_slot)) or wts.numel() < rows * (top + int(shared_slot)):
+            raise RuntimeError("moe_route_sigmoid: ids / wts smaller than rows x choices")
         self.lib.check(self.lib.exl2_moe_route_sigmoid(self._ptr(logits, torch.float32, "logits"), self._ptr(ids, torch.int32, "ids"),
                                                        self._ptr(wts, torch.float32, "wts"), int(rows), int(n_total), int(top), float(scale),
-                                                       self._ptr(gc, torch.int32, "grp_count"), self._ptr(go, torch.int32, "grp_offset"),
+                                                       int(shared_slot), self._ptr(gc, torch.int32, "grp_count"), self._ptr(go, torch.int32, "grp_offset"),
                                                        self._ptr(gr, torch.int32, "grp_rows"), self._stream(logits)))
 
     def wkv_mix(self, h, prev, mu, out, row_seq, row_pos, spans, rows: int, width: int) -> None:

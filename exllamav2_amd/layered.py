@@ -110,6 +110,8 @@ class StepBatch:
     span_chunks: tuple | None = None
     # host-side view of the same rows, one tuple per request in the step: (first row, rows, sequence slot, first position)
     spans: list | None = None
+    # logit_rows is 0 .. rows - 1 in order (every row's logits are wanted, as in decoding): a model may skip the gather
+    logits_all_rows: bool = False
 
 
 class LayeredModel:
@@ -304,12 +306,15 @@ class LayeredModel:
                 norm.forward(x32, pending, xh, rows, dtype=self.dtype)
                 y, mix = module.forward(xh, rows)
                 pending = (y, mix[0], mix[1].shape[-1]) if mix is not None else (y, None, 0)
-        if pending is not None:
-            self.final_norm.forward(x32, pending, None, rows, dtype=self.dtype)
-        if batch.n_logits == 0:
-            return None
-        xn = self.buf("xn", (batch.n_logits, self.width), self.dtype)
-        self.final_norm.forward(x32, None, xn, batch.n_logits, row_idx=batch.logit_rows, dtype=self.dtype)
+        xn = self.buf("xn", (max(batch.n_logits, 1), self.width), self.dtype)
+        if batch.logits_all_rows and batch.n_logits == rows:
+            self.final_norm.forward(x32, pending, xn, rows, dtype=self.dtype)       # the last addition and the final norm in one launch
+        else:
+            if pending is not None:
+                self.final_norm.forward(x32, pending, None, rows, dtype=self.dtype)
+            if batch.n_logits == 0:
+                return None
+            self.final_norm.forward(x32, None, xn, batch.n_logits, row_idx=batch.logit_rows, dtype=self.dtype)
         scaled = cfg.logit_scale != 1.0
         return self.head.forward(xn, batch.n_logits, out=self.buf("logits", (batch.n_logits, self.vocab), f32),
                                  epi=ext.EPI_SCALE if scaled else ext.EPI_NONE, limit=cfg.logit_scale)

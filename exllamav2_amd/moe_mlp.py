@@ -126,7 +126,8 @@ class SigmoidMoEMLP:
     weigh their experts as they are (no renormalisation).  The weight multiplies the expert's INPUT: the token's part is
     sum_e expert_e(s_e h), expert(z) = W_down act(W_up z) with act = relu^2 and no gate matrix; since W_up (s h) = s (W_up h) the
     up projection runs on h and the weight enters in its epilogue, in front of the activation (csrc/dense.hip).  A shared expert of
-    the same form (its own width) runs for every token.  Few rows: every (token, choice) pair names its expert's slab; many rows:
+    the same form (its own width) runs for every token: as wide as the routed ones it is stacked behind them and rides their
+    launches as one more pair per token, otherwise it runs as a two-matrix feed-forward of its own.  Few rows: every (token, choice) pair names its expert's slab; many rows:
     one grouped launch per projection.  forward returns (y | None, mixture): y is the shared expert's output, the chosen experts'
     rows are added by the residual step's launch (rmsnorm.PreShiftRMSNorm)."""
 
@@ -143,40 +144,46 @@ class SigmoidMoEMLP:
         from .mlp import DenseActMLP
         E, width = self.experts, self.model.width
         self.router = DenseLinear(self.ext, self.key + ".router", get("router"))
-        stack = lambda name: torch.stack([get(f"e{e}.{name}") for e in range(E)], 0)
+        # a shared expert as wide as the routed ones is stacked behind them as expert E: the router's launch names it for every token
+        # with weight 1 and the two expert launches run it with the chosen ones
+        self.merged = bool(self.shared_ff) and self.shared_ff == self.ff
+        names = [f"e{e}" for e in range(E)] + (["shared"] if self.merged else [])
+        stack = lambda name: torch.stack([get(f"{n}.{name}") for n in names], 0)
         self.up = DenseLinear(self.ext, self.key + ".up", stack("up"))
         self.down = DenseLinear(self.ext, self.key + ".down", stack("down"))
-        if tuple(self.router.weight.shape) != (E, width) or tuple(self.up.weight.shape) != (E, self.ff, width) \
-                or tuple(self.down.weight.shape) != (E, width, self.ff):
+        self.slabs = len(names)
+        if tuple(self.router.weight.shape) != (E, width) or tuple(self.up.weight.shape) != (self.slabs, self.ff, width) \
+                or tuple(self.down.weight.shape) != (self.slabs, width, self.ff):
             raise RuntimeError(f"{self.key}: tensor shapes do not match the feed-forward's sizes")
         self.shared = None
-        if self.shared_ff:
+        if self.shared_ff and not self.merged:
             self.shared = DenseActMLP(self.model, self.key + ".shared", self.layer_idx).load(lambda n: get("shared." + n))
             if self.shared.up.out_features != self.shared_ff:
                 raise RuntimeError(f"{self.key}: the shared expert is {self.shared.up.out_features} wide, config says {self.shared_ff}")
         return self
 
     def weight_bytes(self) -> int:
-        n = self.router.weight_bytes() + (self.up.weight_bytes() + self.down.weight_bytes()) // self.experts * self.top
+        n = self.router.weight_bytes() + (self.up.weight_bytes() + self.down.weight_bytes()) // self.slabs * (self.top + int(self.merged))
         return n + (self.shared.weight_bytes() if self.shared is not None else 0)
 
     def forward(self, xh: torch.Tensor, rows: int):
         ext, m = self.ext, self.model
         E, top, ff, width, dt = self.experts, self.top, self.ff, m.width, m.dtype
         logits = self.router.forward(xh, rows, out=m.buf("moe.logits", (rows, E), torch.float32))
-        ids = m.buf("moe.ids", (rows, top), torch.int32)
-        wts = m.buf("moe.wts", (rows, top), torch.float32)
-        pairs = rows * top
+        per_row, S = top + int(self.merged), self.slabs          # (token, expert) pairs per row; weight slabs
+        ids = m.buf("moe.ids", (rows, per_row), torch.int32)
+        wts = m.buf("moe.wts", (rows, per_row), torch.float32)
+        pairs = rows * per_row
         grouped = pairs > self.PAIR_ROWS_MAX
         groups = None
         if grouped:
-            groups = (m.buf("moe.count", (E,), torch.int32), m.buf("moe.offset", (E,), torch.int32), m.buf("moe.rows", (pairs,), torch.int32))
-        ext.moe_route_sigmoid(logits, ids, wts, rows, E, top, self.route_scale, groups=groups)
+            groups = (m.buf("moe.count", (S,), torch.int32), m.buf("moe.offset", (S,), torch.int32), m.buf("moe.rows", (pairs,), torch.int32))
+        ext.moe_route_sigmoid(logits, ids, wts, rows, E, top, self.route_scale, groups=groups, shared_slot=self.merged)
         a = m.buf("moe.a", (pairs, ff), dt)
         y = m.buf("moe.y", (pairs, width), torch.float32)
-        kw = dict(batch=E, groups=groups) if grouped else dict(w_sel=ids.view(-1), n_sel=E)
-        ext.dense_linear(xh, self.up.weight, a, pairs, ff, width, width, width, ff, swb=ff * width, x_div=top,
+        kw = dict(batch=S, groups=groups) if grouped else dict(w_sel=ids.view(-1), n_sel=S)
+        ext.dense_linear(xh, self.up.weight, a, pairs, ff, width, width, width, ff, swb=ff * width, x_div=per_row,
                          aux=wts, ldaux=1, epi=ext.EPI_ROW_SCALED_RELU_SQUARED, **kw)
         ext.dense_linear(a, self.down.weight, y, pairs, width, ff, ff, ff, width, swb=width * ff, **kw)
         ys = self.shared.forward(xh, rows)[0] if self.shared is not None else None
-        return ys, (y, ids, wts, E)
+        return ys, (y, ids, wts, S)

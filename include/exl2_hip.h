@@ -555,9 +555,11 @@ int exl2_add_rms_shift(float* x, const float* y, const float* moe_y, int top, fl
 int exl2_span_last_rows(const float* src, int ld, float* slot_rows, int width, const int* span_row0, const int* span_rows,
                         int spans, const int* row_seq, void* stream);
 /* router with independent scores: score = sigmoid(logit); the `top` largest are chosen (first index on a tie); weight = score *
-   scale, not renormalised.  grp_* as in exl2_moe_route_scored. */
+   scale, not renormalised.  shared_slot: ids / wts are [rows, top + 1] and the last column names expert n_total with weight 1 (an
+   expert every token uses, stacked behind the routed ones so that one launch runs both).  grp_* as in exl2_moe_route_scored, over
+   n_total (+ 1) experts. */
 int exl2_moe_route_sigmoid(const float* logits, int* ids, float* wts, int rows, int n_total, int top, float scale,
-                           int* grp_count, int* grp_offset, int* grp_rows, void* stream);
+                           int shared_slot, int* grp_count, int* grp_offset, int* grp_rows, void* stream);
 
 /* ---- linear attention with a per-channel data-dependent decay (csrc/wkv.hip) */
 

@@ -115,26 +115,30 @@ def test_dense_linear_scale_tanh_and_row_scaled_activation(be, dtype, M, N, K, e
     assert close(be.n(y), want, 2e-5)
 
 
-@pytest.mark.parametrize("experts,top", [(5, 1), (5, 2), (16, 1), (70, 4), (3, 3)])
-def test_sigmoid_router_and_expert_lists(be, experts, top):
+@pytest.mark.parametrize("shared", [False, True])
+@pytest.mark.parametrize("experts,top", [(5, 1), (5, 2), (12, 1), (70, 4), (3, 3)])
+def test_sigmoid_router_and_expert_lists(be, experts, top, shared):
+    """shared: one more column per row names the expert behind the routed ones, weight 1, and the lists have one more expert"""
     rng = np.random.default_rng(experts * 10 + top)
-    rows = 37
+    rows, per = 37, top + int(shared)
     logits = rng.standard_normal((rows, experts)).astype(np.float32) * 2
     logits[3, :] = 0.25                                          # a tie over all experts: the lowest indices win
-    ids = torch.zeros((rows, top), dtype=I32, device=be.device)
-    wts = torch.zeros((rows, top), dtype=F32, device=be.device)
-    groups = tuple(torch.zeros((n,), dtype=I32, device=be.device) for n in (experts, experts, rows * top))
-    be.ext.moe_route_sigmoid(be.t(logits), ids, wts, rows, experts, top, groups=groups)
+    ids = torch.zeros((rows, per), dtype=I32, device=be.device)
+    wts = torch.zeros((rows, per), dtype=F32, device=be.device)
+    groups = tuple(torch.zeros((n,), dtype=I32, device=be.device) for n in (experts + 1, experts + 1, rows * per))
+    be.ext.moe_route_sigmoid(be.t(logits), ids, wts, rows, experts, top, groups=groups, shared_slot=shared)
     gi, gw = be.n(ids), be.n(wts)
     for r in range(rows):
         s = ON.sigmoid(logits[r].astype(np.float64))
         order = sorted(range(experts), key=lambda e: (-s[e], e))[:top]
-        assert list(gi[r]) == order, r
-        assert close(gw[r], s[order], 1e-6)
+        assert list(gi[r][:top]) == order, r
+        assert close(gw[r][:top], s[order], 1e-6)
+        if shared:
+            assert gi[r][top] == experts and gw[r][top] == 1.0
     cnt, off, lst = (be.n(t) for t in groups)
     flat = gi.reshape(-1)
-    for e in range(experts):
-        mine = [p for p in range(rows * top) if flat[p] == e]
+    for e in range(experts + int(shared)):
+        mine = [p for p in range(rows * per) if flat[p] == e]
         assert cnt[e] == len(mine) and list(lst[off[e]:off[e] + cnt[e]]) == mine
 
 
@@ -148,7 +152,7 @@ def attention_case(be, dtype, H, G, dim, vd, chunk, page, lens_by_step, softcap,
     rng = np.random.default_rng(seed)
     width = 24
     m = ON.attn_mixer(heads=H, kv_heads=G, dim=dim, vdim=vd, size=chunk, dims=rot_dims, softcap=softcap,
-                      scaling={"factor": 4.0, "original": 32, "low": 1.0, "high": 4.0})["mixer"]
+                      scaling={"factor": 3.0, "original": 40, "low": 2.0, "high": 8.0})["mixer"]
     W = {"l0.mix." + n: ON.bf16_round(rng.standard_normal(s) / math.sqrt(width) * g)
          for n, s, g in (("q", (H * dim, width), 3.0), ("k", (G * dim, width), 3.0), ("v", (G * vd, width), 1.0), ("g", (H, width), 2.0))}
     W["l0.mix.o"] = np.eye(H * vd)
