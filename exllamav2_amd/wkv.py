@@ -4,7 +4,8 @@ Per token, with h the mixer's input and h' the previous token's input (zeros at 
     x_s = h + (h' - h) * mu_s                          five blends, s in (r, k, v, g, w)                (csrc/wkv.hip: wkv_mix_kernel)
     r, k, v = W_r x_r, W_k x_k, W_v x_v                heads x dim each;   gate = silu(W_g x_g)
     d = W_w2 tanh(W_w1 x_w) + w0;  w = exp(-exp(d))    decay per head and key channel, in (0, 1)
-    head i:  o = (S_i + diag(u_i) k v^T)^T r;  S_i <- diag(w) S_i + k v^T        S fp32 [dim, dim] per slot  (wkv_scan_kernel)
+    head i:  o = (S_i + diag(u_i) k v^T)^T r;  S_i <- diag(w) S_i + k v^T        S fp32 [dim, dim] per slot  (wkv_scan_kernel token by
+             token for decoded tokens and short portions; wkv_chunk_* unrolled in chunks of 64 tokens for portions of prompts)
     out = W_o (o / rms_per_head(o) * norm * gate)
 Between steps a sequence keeps S and its last input row in its slot (cache.SlotState).  The mixer reads its input in fp32
 (`input_f32`): the blends are rounded to the operand dtype once, after blending.  Head count, head size and the rank of the decay's
