@@ -139,6 +139,13 @@ PROTOTYPES = {
     "exl2_wkv_scan": (ci, [vp, vp, vp, vp, ci, vp, ci, vp, vp, vp, ci, ci, vp, vp, vp, ci, vp, vp, ci, ci, ci, cf, vp]),
     "exl2_wkv_scan_chunked_supported": (ci, [ci, ci]),
     "exl2_wkv_scan_chunked": (ci, [vp, vp, vp, vp, ci, vp, ci, vp, vp, vp, ci, ci, vp, vp, vp, vp, ci, ci, ci, vp, vp, vp, vp, ci, ci, ci, cf, vp]),
+    # sandwich-normed residual step, token-pair embedding (csrc/rowops.hip); convolution variants (csrc/ssm.hip); matrix-state recurrences
+    # (csrc/gated_scan.hip)
+    "exl2_sandwich_norm": (ci, [vp, vp, cf, vp, cf, vp, ci, vp, cf, vp, vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, cf, vp]),
+    "exl2_embed_pair": (ci, [vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, vp, ci, ci, ci, ci, ci, ci, ci, cf, ci, cf, vp]),
+    "exl2_conv_rows_ex": (ci, [vp, ci, vp, vp, vp, ci, ci, ci, vp, vp, vp, ci, ci, vp, vp, ci, ci, ci, vp]),
+    "exl2_gated_scan": (ci, [ci, vp, ci, vp, ci, vp, ci, vp, ci, vp, ci, vp, ci, vp, vp, vp, vp, vp, ci, ci, vp, vp, vp, ci, vp, vp, ci, ci,
+                             ci, ci, cf, cf, vp]),
     # graphs
     "exl2_graph_begin_capture": (ci, [vp]),
     "exl2_graph_end_capture": (ci, [vp, C.POINTER(vp)]),

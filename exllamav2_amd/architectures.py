@@ -57,6 +57,7 @@ def _build_quantized(cfg, tensors, device, dtype, ext):
 register("Benolix", LayeredConfig.from_dict, _build_layered)
 register("Tibalorn", LayeredConfig.from_dict_prenorm, _build_layered)
 register("Negilorn", LayeredConfig.from_dict_prerms_shift, _build_layered)
+register("Kilurax", LayeredConfig.from_dict_sandwich, _build_layered)
 register("LlamaForCausalLM", _read_llama, _build_quantized)
 register("MixtralForCausalLM", _read_llama, _build_quantized)
 

@@ -10,8 +10,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libexl2_hip.so")
 # What the unquantized (dense-weight) models need -- their kernels, the checkpoint reader, the sampler, graphs -- as a library of its
-# own: a fresh checkout that only ever serves such a model compiles these ten sources (about a minute) instead of the whole tree.
-DENSE_SOURCES = ("errors", "dense", "rowops", "latent_attn", "ssm", "window_attn", "wkv", "stloader", "sampling", "graph")
+# own: a fresh checkout that only ever serves such a model compiles these eleven sources (about a minute) instead of the whole tree.
+DENSE_SOURCES = ("errors", "dense", "rowops", "latent_attn", "ssm", "window_attn", "wkv", "gated_scan", "stloader", "sampling", "graph")
 OUT_DENSE = os.path.join(HERE, "libexl2_hip_dense.so")
 
 

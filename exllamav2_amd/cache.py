@@ -197,11 +197,12 @@ class PagedKV:
 
 
 class SlotState:
-    """One recurrent layer's state per sequence slot of a PagePool: named fp32 tensors [max_seqs, ...].  Nothing is cleared when a
-    slot is handed to a new sequence: the kernels start a sequence's first portion (position 0) from zeros by themselves."""
+    """One recurrent layer's state per sequence slot of a PagePool: named tensors [max_seqs, ...], fp32 unless `dtype` says otherwise
+    (int32 for remembered tokens).  Nothing is cleared when a slot is handed to a new sequence: the kernels start a sequence's first
+    portion (position 0) from zeros by themselves."""
 
-    def __init__(self, pool: PagePool, shapes: dict):
-        self.t = {name: torch.zeros((pool.max_seqs,) + tuple(shape), dtype=torch.float32, device=pool.device)
+    def __init__(self, pool: PagePool, shapes: dict, dtype=torch.float32):
+        self.t = {name: torch.zeros((pool.max_seqs,) + tuple(shape), dtype=dtype, device=pool.device)
                   for name, shape in shapes.items()}
 
     def __getitem__(self, name: str) -> torch.Tensor:
@@ -218,13 +219,16 @@ class LayerStates:
 
     def __init__(self, pool: PagePool, per_layer: dict, norm_states: dict | None = None):
         self.pool, self.per_layer = pool, dict(per_layer)
-        self.norm_states = dict(norm_states or {})            # layer -> what the norm in front of its mixer keeps per slot (token shift)
+        # what the row-wise steps keep per slot: layer -> the norm in front of its mixer (token shift, input convolution),
+        # (layer, "ff") -> the norm in front of its feed-forward, "embed" -> the embedding (previous token)
+        self.norm_states = dict(norm_states or {})
 
-    def layer(self, layer_idx: int):
-        return self.per_layer[layer_idx]
+    def layer(self, key):
+        """key: a layer's index, or whatever a mixer that keeps several states names them by"""
+        return self.per_layer[key]
 
-    def norm_state(self, layer_idx: int):
-        return self.norm_states.get(layer_idx)
+    def norm_state(self, key):
+        return self.norm_states.get(key)
 
     def footprint(self) -> int:
         states = list(self.per_layer.values()) + list(self.norm_states.values())

@@ -70,6 +70,12 @@ class LayeredConfig:
     logit_softcap: float = 0.0        # > 0: logits <- c tanh(logits / c)
     logit_scale: float = 1.0          # logits <- logits * s
     attention_mask: str = "window"    # what an attention layer's mask.size means: "window" (sliding) or "chunk" (blocks from position 0)
+    # "sandwich": x <- x + residual_mult * n_g(f(conv_in(n_g(x) w_in))) w_out with RMS norms over `norm_groups` equal runs of the row and
+    # a causal convolution of `input_conv_taps` taps beside the identity in front of every sublayer (0: none)
+    norm_groups: int = 1
+    residual_mult: float = 1.0
+    input_conv_taps: int = 0
+    pair_embedding: dict | None = None   # {"buckets", "mul_prev", "mul_cur"}: a hashed (previous token, token) table added to the embedding
 
     @staticmethod
     def from_dict_prenorm(d: dict) -> "LayeredConfig":
@@ -96,6 +102,29 @@ class LayeredConfig:
             raise RuntimeError(f"config.json: missing key {e}") from e
         if cfg.vocab <= 0 or cfg.width <= 0 or not cfg.layers:
             raise RuntimeError("config.json: vocab, width and layers must be given")
+        return cfg
+
+    @staticmethod
+    def from_dict_sandwich(d: dict) -> "LayeredConfig":
+        """stacks whose sublayers stand between two grouped RMS norms behind a short input convolution, with a scaled residual branch,
+        a token-pair table beside the embedding and a `head` matrix"""
+        try:
+            emb = d["embedding"]
+            pair = emb.get("bigram")
+            cfg = LayeredConfig(architecture=str(d["architecture"]), vocab=int(d["vocab"]), width=int(d["width"]),
+                                norm_eps=float(d["norm"]["eps"]), norm_groups=int(d["norm"].get("groups", 1)),
+                                embedding_scale=float(emb.get("scale", 1.0)), layers=list(d["layers"]), residual="sandwich",
+                                residual_mult=float(d.get("residual_mult", 1.0)), input_conv_taps=int((d.get("canon") or {}).get("taps", 0)),
+                                pair_embedding=({"buckets": int(pair["buckets"]), "mul_prev": int(pair["mul_prev"]),
+                                                 "mul_cur": int(pair["mul_cur"])} if pair else None))
+        except KeyError as e:
+            raise RuntimeError(f"config.json: missing key {e}") from e
+        if cfg.vocab <= 0 or cfg.width <= 0 or not cfg.layers:
+            raise RuntimeError("config.json: vocab, width and layers must be given")
+        if cfg.norm_groups <= 0 or cfg.width % cfg.norm_groups:
+            raise RuntimeError(f"config.json: {cfg.width} values do not split into {cfg.norm_groups} norm groups")
+        if cfg.pair_embedding is not None and cfg.pair_embedding["buckets"] <= 0:
+            raise RuntimeError("config.json: the token-pair table needs a positive number of buckets")
         return cfg
 
     @staticmethod

@@ -14,15 +14,17 @@
 // Epilogues fold the layer's elementwise steps into the producing linear: acc * sigmoid(aux) (output gate), silu(aux) * acc
 // (gated MLP), the clamped gated unit min(aux, L) * sigmoid(1.702 min(aux, L)) * (clamp(acc, -L, L) + 1), relu(acc)^2, the soft
 // cap L tanh(acc / L), a plain scale L acc, tanh(acc), and relu(aux[row] acc)^2 (an expert whose INPUT carries the router's weight:
-// W (s h) = s (W h)); a bias vector (fp32, one value per output column) is added to the accumulator first.
+// W (s h) = s (W h)), the two halves of a gated unit on such an input -- silu(aux[row] acc) aux[row] from the gate matrix, then
+// aux acc from the up matrix --; a bias vector (fp32, one value per output column) is added to the accumulator first.
 #include "hw.h"
 #include "errors.h"
 
 enum { DENSE_BF16 = 0, DENSE_F32 = 1 };
 enum { EPI_NONE = 0, EPI_MUL_SIGMOID_AUX = 1, EPI_SILU_AUX_MUL = 2, EPI_CLAMPED_GLU = 3, EPI_RELU_SQUARED = 4, EPI_SOFT_CAP = 5,
-       EPI_SCALE = 6, EPI_TANH = 7, EPI_ROW_SCALED_RELU_SQUARED = 8, EPI_LAST = 8 };
-#define EPI_ROW_AUX(e) ((e) == EPI_ROW_SCALED_RELU_SQUARED)          // aux holds ONE value per row (ldaux apart), not one per output
-#define EPI_READS_AUX(e) (((e) >= EPI_MUL_SIGMOID_AUX && (e) <= EPI_CLAMPED_GLU) || EPI_ROW_AUX(e))
+       EPI_SCALE = 6, EPI_TANH = 7, EPI_ROW_SCALED_RELU_SQUARED = 8, EPI_ROW_SCALED_SILU_SCALED = 9, EPI_AUX_MUL = 10, EPI_LAST = 10 };
+// aux holds ONE value per row (ldaux apart), not one per output
+#define EPI_ROW_AUX(e) ((e) == EPI_ROW_SCALED_RELU_SQUARED || (e) == EPI_ROW_SCALED_SILU_SCALED)
+#define EPI_READS_AUX(e) (((e) >= EPI_MUL_SIGMOID_AUX && (e) <= EPI_CLAMPED_GLU) || EPI_ROW_AUX(e) || (e) == EPI_AUX_MUL)
 #define EPI_AUX_COL(e, n) (EPI_ROW_AUX(e) ? 0 : (n))
 
 struct LinArgs
@@ -85,6 +87,8 @@ DEV float lin_epilogue(int epi, float acc, float aux, float limit)
     if (epi == EPI_SCALE) return acc * limit;
     if (epi == EPI_TANH) return tanhf(acc);
     if (epi == EPI_ROW_SCALED_RELU_SQUARED) { const float r = fmaxf(acc * aux, 0.0f); return r * r; }
+    if (epi == EPI_ROW_SCALED_SILU_SCALED) { const float z = acc * aux; return z * sigmoid_f32(z) * aux; }
+    if (epi == EPI_AUX_MUL) return acc * aux;
     return acc;
 }
 

@@ -1,0 +1,257 @@
+// gated_scan.hip -- two linear-attention recurrences over a matrix state per head, for gfx950, + their C ABI.
+//
+// Per head, with the state S (N key channels x P value channels, fp32, one per (slot, head)):
+//   mode 0, "forget gate writes":   f = l + (1 - l) sigmoid(z_f)  per key channel (l = a learned lower bound),  q = silu(z_q),
+//       S <- diag(f) S + (1 - f) v^T,    o = S^T q;
+//   mode 1, "gated delta rule":     q, k made unit vectors per head (x / sqrt(sum x^2 + 1e-6)), q also times q_scale,
+//       beta = sigmoid(z_b),  g = exp(-exp(A) softplus(z_a + a_bias))  (one number per head),
+//       S <- g S,   u = beta (v - S^T k),   S <- S + k u^T,   o = S^T q        (the read-out sees the token's own write).
+// The head's o is divided by its root mean square over P, multiplied by a weight per value channel (shared by the heads) and, in
+// mode 1, by silu of an output gate, and leaves in the operand dtype for the output projection.  Query / key heads may be fewer than
+// value heads (head h reads q / k head h / (heads / qk_heads)).  Inputs are the fp32 outputs of the mixer's projections (mode 1: of
+// its short convolutions); gates, decays, unit norms and the state are fp32 throughout.
+//
+// Rows of a step are a flat list; a span is the run of consecutive rows one sequence brings (span i = rows span_row0[i] ..
+// + span_rows[i], slot and first position = row_seq / row_pos of its first row).  A span at position 0 starts from zeros whatever
+// its slot holds.
+#include "hw.h"
+#include "errors.h"
+#include <stdint.h>
+
+template <typename T> DEV void gs_st(T* p, float v);
+template <> DEV void gs_st<u16>(u16* p, float v) { *p = f32_to_bf16(v); }
+template <> DEV void gs_st<float>(float* p, float v) { *p = v; }
+
+DEV float gs_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
+DEV float gs_softplus(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+
+#define GS_CHUNK 16                          // tokens staged in LDS per round
+#define GS_MAX_NPT 256                       // state rows per thread
+#define GS_MAX_N 1024                        // key channels per head (16 per lane while a wave normalises a token's q and k)
+
+enum { GS_FORGET_WRITES = 0, GS_DELTA = 1 };
+
+struct GatedScanArgs
+{
+    const float* q; int ldq;                 // [rows, ldq]: q head g at g * N (mode 0: pre-activation)
+    const float* k; int ldk;                 // mode 1: keys, head g at g * N;  mode 0: the forget gate's pre-activation, head h at h * N
+    const float* v; int ldv;                 // head h at h * P
+    const float* gate; int ldg;              // mode 1: output gate pre-activation, head h at h * P (nullable)
+    const float* beta; int ldb;              // mode 1: [rows, ldb], head h at h (pre-sigmoid)
+    const float* dt; int lddt;               // mode 1: [rows, lddt], head h at h
+    const float* dt_bias; const float* a_log;        // mode 1: [heads]
+    const float* lower;                      // mode 0: [heads * N]
+    const float* norm_w;                     // [P]
+    void* out; int ldo;                      // [rows, ldo] operand dtype (or fp32): head h at h * P
+    float* state;                            // [slots, heads, N, P]
+    const int* span_row0; const int* span_rows; const int* row_seq; const int* row_pos;
+    int heads, qk_heads, N, P, KS;           // KS (a power of two <= 64) lanes share a column of the state
+    float q_scale, eps;
+};
+
+// Workgroup = one (span, head): thread t = p * KS + j holds rows n = j, j + KS, .. of column p of the state in registers for the whole
+// span; the KS lanes of a column are neighbours in one wave, so the two sums over key channels that a token needs (S^T k for the delta
+// rule, S^T q for the read-out) close with lane exchanges, no barrier.  Tokens are taken GS_CHUNK at a time: a wave per token turns
+// the raw projections into what the recurrence reads (gates, unit vectors, decay) and stages it in LDS, every thread steps its rows
+// through the chunk, and a wave per token takes the head's root mean square and writes the normed (gated) row.
+template <typename T, int NPT, int MODE>
+KERNEL void __launch_bounds__(256) gated_scan_kernel(const GatedScanArgs a)
+{
+    DYN_SMEM(smem);
+    const int h = bid_x(), sp = bid_y();
+    const int n_tok = a.span_rows[sp], r0 = a.span_row0[sp];
+    const int pos0 = a.row_pos[r0];
+    const int P = a.P, N = a.N, KS = a.KS;
+    const int t = tid(), nt = nthreads();
+    const bool owner = t < P * KS;
+    const int p = owner ? t / KS : 0, j = t % KS;
+    const int hq = h / (a.heads / a.qk_heads);
+    float* s_q = (float*)smem;                                   // [CHUNK, N]
+    float* s_k = s_q + GS_CHUNK * N;                             // [CHUNK, N]  mode 1: unit keys; mode 0: forget gates
+    float* s_v = s_k + GS_CHUNK * N;                             // [CHUNK, P]
+    float* s_o = s_v + GS_CHUNK * P;                             // [CHUNK, P]
+    float* s_b = s_o + GS_CHUNK * P;                             // [CHUNK] beta
+    float* s_g = s_b + GS_CHUNK;                                 // [CHUNK] decay
+    float* st = a.state + ((long long)a.row_seq[r0] * a.heads + h) * (long long)N * P;
+    float S[NPT];
+    #pragma unroll
+    for (int i = 0; i < NPT; i++)
+    {
+        const int n = j + KS * i;
+        S[i] = (owner && pos0 > 0 && n < N) ? st[(long long)n * P + p] : 0.0f;
+    }
+    for (int c0 = 0; c0 < n_tok; c0 += GS_CHUNK)
+    {
+        const int nc = min(GS_CHUNK, n_tok - c0);
+        block_sync();
+        for (int kk = wave_id(); kk < nc; kk += nt / 64)
+        {
+            const long long row = r0 + c0 + kk;
+            if (MODE == GS_DELTA)
+            {
+                float qv[GS_MAX_N / 64], kv[GS_MAX_N / 64];
+                float sq = 0.0f, sk = 0.0f;
+                #pragma unroll
+                for (int e = 0; e < GS_MAX_N / 64; e++)
+                {
+                    const int n = lane_id() + 64 * e;
+                    qv[e] = n < N ? a.q[row * a.ldq + hq * N + n] : 0.0f;
+                    kv[e] = n < N ? a.k[row * a.ldk + hq * N + n] : 0.0f;
+                    sq = fmaf(qv[e], qv[e], sq);
+                    sk = fmaf(kv[e], kv[e], sk);
+                }
+                sq = wave_allreduce_add(sq);
+                sk = wave_allreduce_add(sk);
+                const float mq = a.q_scale / sqrtf(sq + 1e-6f), mk = 1.0f / sqrtf(sk + 1e-6f);
+                #pragma unroll
+                for (int e = 0; e < GS_MAX_N / 64; e++)
+                {
+                    const int n = lane_id() + 64 * e;
+                    if (n < N) { s_q[kk * N + n] = qv[e] * mq; s_k[kk * N + n] = kv[e] * mk; }
+                }
+                if (lane_id() == 0)
+                {
+                    s_b[kk] = gs_sigmoid(a.beta[row * a.ldb + h]);
+                    s_g[kk] = expf(-expf(a.a_log[h]) * gs_softplus(a.dt[row * a.lddt + h] + a.dt_bias[h]));
+                }
+            }
+            else
+            {
+                for (int n = lane_id(); n < N; n += 64)
+                {
+                    const float zq = a.q[row * a.ldq + h * N + n];
+                    const float lo = a.lower[h * N + n];
+                    s_q[kk * N + n] = zq * gs_sigmoid(zq);
+                    s_k[kk * N + n] = fmaf(1.0f - lo, gs_sigmoid(a.k[row * a.ldk + h * N + n]), lo);
+                }
+            }
+            for (int pp = lane_id(); pp < P; pp += 64) s_v[kk * P + pp] = a.v[row * a.ldv + h * P + pp];
+        }
+        block_sync();
+        for (int kk = 0; kk < nc; kk++)
+        {
+            const float vv = s_v[kk * P + p];
+            float o = 0.0f;
+            if (MODE == GS_DELTA)
+            {
+                const float g = s_g[kk];
+                float kt = 0.0f;
+                #pragma unroll
+                for (int i = 0; i < NPT; i++)
+                {
+                    const int n = j + KS * i;
+                    if (n < N) { S[i] *= g; kt = fmaf(S[i], s_k[kk * N + n], kt); }
+                }
+                for (int m = 1; m < KS; m <<= 1) kt += shfl_xor_f32(kt, m);
+                const float u = s_b[kk] * (vv - kt);
+                #pragma unroll
+                for (int i = 0; i < NPT; i++)
+                {
+                    const int n = j + KS * i;
+                    if (n < N) { S[i] = fmaf(s_k[kk * N + n], u, S[i]); o = fmaf(S[i], s_q[kk * N + n], o); }
+                }
+            }
+            else
+            {
+                #pragma unroll
+                for (int i = 0; i < NPT; i++)
+                {
+                    const int n = j + KS * i;
+                    if (n < N)
+                    {
+                        const float f = s_k[kk * N + n];
+                        S[i] = fmaf(f, S[i], (1.0f - f) * vv);
+                        o = fmaf(S[i], s_q[kk * N + n], o);
+                    }
+                }
+            }
+            for (int m = 1; m < KS; m <<= 1) o += shfl_xor_f32(o, m);
+            if (owner && j == 0) s_o[kk * P + p] = o;
+        }
+        block_sync();
+        for (int kk = wave_id(); kk < nc; kk += nt / 64)
+        {
+            float ss = 0.0f;
+            for (int pp = lane_id(); pp < P; pp += 64) { const float ov = s_o[kk * P + pp]; ss = fmaf(ov, ov, ss); }
+            ss = wave_allreduce_add(ss);
+            const float rinv = 1.0f / sqrtf(ss / (float)P + a.eps);
+            const long long row = r0 + c0 + kk;
+            for (int pp = lane_id(); pp < P; pp += 64)
+            {
+                float o = s_o[kk * P + pp] * rinv * a.norm_w[pp];
+                if (a.gate) { const float gv = a.gate[row * a.ldg + h * P + pp]; o *= gv * gs_sigmoid(gv); }
+                gs_st<T>((T*)a.out + row * a.ldo + h * P + pp, o);
+            }
+        }
+    }
+    #pragma unroll
+    for (int i = 0; i < NPT; i++)
+    {
+        const int n = j + KS * i;
+        if (owner && n < N) st[(long long)n * P + p] = S[i];
+    }
+}
+
+template <typename T, int MODE>
+static void gated_scan_launch(const GatedScanArgs& a, int npt, dim3 grid, dim3 block, size_t smem, void* stream)
+{
+    if (npt <= 16) LAUNCH((gated_scan_kernel<T, 16, MODE>), grid, block, smem, stream, a);
+    else if (npt <= 64) LAUNCH((gated_scan_kernel<T, 64, MODE>), grid, block, smem, stream, a);
+    else LAUNCH((gated_scan_kernel<T, GS_MAX_NPT, MODE>), grid, block, smem, stream, a);
+}
+
+/* The recurrence over the rows of every span, state read from and left in state[slot of the span][head].  mode 0: k is the forget
+   gate's pre-activation (heads x n_key), lower its lower bound, qk_heads == heads; gate / beta / dt / dt_bias / a_log unused.
+   mode 1: q / k hold qk_heads heads, beta / dt one value per head, gate nullable; lower unused.  All inputs fp32. */
+extern "C" int exl2_gated_scan(int mode, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* gate,
+                               int ldg, const float* beta, int ldb, const float* dt, int lddt, const float* dt_bias, const float* a_log,
+                               const float* lower, const float* norm_w, void* out, int ldo, int out_f32, float* state,
+                               const int* span_row0, const int* span_rows, int spans, const int* row_seq, const int* row_pos, int heads,
+                               int qk_heads, int n_key, int n_val, float q_scale, float eps, void* stream)
+{
+    EXL2_REQUIRE(mode == GS_FORGET_WRITES || mode == GS_DELTA, "gated_scan: mode must be 0 (forget gate writes) or 1 (delta rule)");
+    EXL2_REQUIRE(q && k && v && norm_w && out && state && span_row0 && span_rows && row_seq && row_pos, "gated_scan: null operand");
+    EXL2_REQUIRE(mode != GS_FORGET_WRITES || lower, "gated_scan: the forget gate needs its lower bound");
+    EXL2_REQUIRE(mode != GS_DELTA || (beta && dt && dt_bias && a_log), "gated_scan: the delta rule needs beta and the decay's inputs");
+    EXL2_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && (mode == GS_DELTA || qk_heads == heads), "gated_scan: %d heads over %d query / key heads", heads, qk_heads);
+    EXL2_REQUIRE(n_key > 0 && n_key <= GS_MAX_N && n_val > 0 && n_val <= 256, "gated_scan: state %d x %d", n_key, n_val);
+    if (spans <= 0) return EXL2_OK;
+    int ks = 1;
+    while (ks * 2 <= 64 && n_val * ks * 2 <= 256 && ks * 2 <= n_key) ks *= 2;
+    const int npt = (n_key + ks - 1) / ks;
+    EXL2_REQUIRE(npt <= GS_MAX_NPT, "gated_scan: state %d x %d needs %d rows per thread (at most %d)", n_key, n_val, npt, GS_MAX_NPT);
+    GatedScanArgs a;
+    a.q = q; a.ldq = ldq; a.k = k; a.ldk = ldk; a.v = v; a.ldv = ldv; a.gate = gate; a.ldg = ldg; a.beta = beta; a.ldb = ldb; a.dt = dt;
+    a.lddt = lddt; a.dt_bias = dt_bias; a.a_log = a_log; a.lower = lower; a.norm_w = norm_w; a.out = out; a.ldo = ldo; a.state = state;
+    a.span_row0 = span_row0; a.span_rows = span_rows; a.row_seq = row_seq; a.row_pos = row_pos;
+    a.heads = heads; a.qk_heads = qk_heads; a.N = n_key; a.P = n_val; a.KS = ks; a.q_scale = q_scale; a.eps = eps;
+    const size_t smem = sizeof(float) * ((size_t)GS_CHUNK * (2 * n_key + 2 * n_val + 2));
+    if (smem > 48 * 1024)
+    {
+        static bool attr_done[EXL2_MAX_DEVICES];
+        if (exl2_first_on_device(attr_done))
+        {
+            (void)hipFuncSetAttribute((const void*)gated_scan_kernel<u16, GS_MAX_NPT, GS_FORGET_WRITES>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_kernel<float, GS_MAX_NPT, GS_FORGET_WRITES>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_kernel<u16, GS_MAX_NPT, GS_DELTA>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_kernel<float, GS_MAX_NPT, GS_DELTA>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_kernel<u16, 64, GS_FORGET_WRITES>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_kernel<float, 64, GS_FORGET_WRITES>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_kernel<u16, 64, GS_DELTA>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_kernel<float, 64, GS_DELTA>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        }
+    }
+    const dim3 grid(heads, spans), block((n_val * ks + 63) / 64 * 64);
+    if (mode == GS_DELTA)
+    {
+        if (out_f32) gated_scan_launch<float, GS_DELTA>(a, npt, grid, block, smem, stream);
+        else gated_scan_launch<u16, GS_DELTA>(a, npt, grid, block, smem, stream);
+    }
+    else
+    {
+        if (out_f32) gated_scan_launch<float, GS_FORGET_WRITES>(a, npt, grid, block, smem, stream);
+        else gated_scan_launch<u16, GS_FORGET_WRITES>(a, npt, grid, block, smem, stream);
+    }
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}

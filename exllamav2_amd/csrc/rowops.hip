@@ -6,6 +6,9 @@
 //     token's chosen experts (identity experts contribute the token's own x),
 //   * the pre-norm residual step  x <- x + y (+ the sum of a token's expert outputs)  with an RMS norm whose gain is ONE number and
 //     a token shift  h + (h' - h) * shift  towards the previous token's normed row (kept per sequence slot),
+//   * the sandwich-normed residual step  x <- x + mult n_g(sublayer) w_out  with the grouped RMS norm  n_g(x) w_in  that feeds the next
+//     sublayer (and, for single-token steps, the short convolution over the last normed rows of the sequence),
+//   * a token embedding plus a hashed (previous token, token) embedding under a grouped RMS norm (the previous token kept per slot),
 //   * the sparse-MoE router (softmax over all experts, selection by score + correction, weights from the uncorrected scores; or
 //     sigmoid scores, selection and weights by the scores themselves) and the per-expert row lists the grouped linear reads.
 // Element type T of weights / operand copies: u16 = bfloat16 bits, float.
@@ -317,6 +320,160 @@ KERNEL void __launch_bounds__(256) span_last_row_kernel(const float* src, int ld
     slot_rows[(long long)row_seq[last] * width + i] = src[(long long)last * ld + i];
 }
 
+// ---- sandwich-normed residual step ---------------------------------------------------------------------------------------------
+// n_g(v) = v cut into `groups` equal runs, each divided by sqrt(mean(run^2) + eps).  One launch per row does
+//     x <- x + mult * n_g(t) w_out,   t = ya y + yb y2 + the sum of the row's `top` expert rows      (any of the three may be absent)
+//     hn = n_g(x) w_in                                                                              (w_in nullable: only the addition)
+// i.e. the norm BEHIND a sublayer, the residual addition and the norm IN FRONT of the next sublayer.  The consumer of hn may read it
+// through a short causal convolution over the sequence, out = hn + sum_j c[:, j] hn_(p - taps + 1 + j): steps whose spans are single
+// rows (decoding) do that here too, from the slot's tail [slots, taps - 1, width] of the last normed rows, and roll the tail (a thread
+// reads and writes only its own channels); otherwise hn goes out in fp32 and the convolution is exl2_conv_rows_ex's.
+
+struct SandwichArgs
+{
+    float* x;
+    const float* y; float ya; const float* y2; float yb; const float* moe_y; int top;
+    const void* w_out; float mult;
+    const void* w_in;
+    void* out; int out_f32;
+    const int* row_idx;                      // nullable: output row r is made from stream row row_idx[r] (no addition then)
+    const void* conv_w; float* tail; const int* row_seq; const int* row_pos; int taps;      // conv_w nullable
+    int width, groups; float eps;
+};
+
+template <typename T>
+KERNEL void __launch_bounds__(256) sandwich_norm_kernel(const SandwichArgs a)
+{
+    DYN_SMEM(smem);
+    SHARED float part[4];
+    float* v = (float*)smem;
+    const int r = bid_x();
+    const long long src = a.row_idx ? a.row_idx[r] : r;
+    float* xr = a.x + src * a.width;
+    const int gs = a.width / a.groups;
+    if (a.y || a.y2 || a.moe_y)
+    {
+        for (int i = tid(); i < a.width; i += 256)
+        {
+            float t = 0.0f;
+            if (a.y) t = a.ya * a.y[src * a.width + i];
+            if (a.y2) t = fmaf(a.yb, a.y2[src * a.width + i], t);
+            for (int k = 0; k < (a.moe_y ? a.top : 0); k++) t += a.moe_y[(src * a.top + k) * a.width + i];
+            v[i] = t;
+        }
+        for (int g = 0; g < a.groups; g++)
+        {
+            float ss = 0.0f;
+            for (int i = g * gs + tid(); i < (g + 1) * gs; i += 256) ss = fmaf(v[i], v[i], ss);
+            ss = block_sum_256(ss, part);
+            const float mul = a.mult / sqrtf(ss / (float)gs + a.eps);
+            for (int i = g * gs + tid(); i < (g + 1) * gs; i += 256)
+            {
+                const float xv = fmaf(v[i] * mul, ro_ld<T>((const T*)a.w_out + i), xr[i]);
+                xr[i] = xv;
+                v[i] = xv;
+            }
+        }
+    }
+    else
+        for (int i = tid(); i < a.width; i += 256) v[i] = xr[i];
+    if (!a.out) return;
+    const bool conv = a.conv_w != nullptr && a.taps > 1;
+    float* tl = nullptr; int pos = 0;
+    if (conv) { tl = a.tail + (long long)a.row_seq[r] * (a.taps - 1) * a.width; pos = a.row_pos[r]; }
+    for (int g = 0; g < a.groups; g++)
+    {
+        float ss = 0.0f;
+        for (int i = g * gs + tid(); i < (g + 1) * gs; i += 256) ss = fmaf(v[i], v[i], ss);
+        ss = block_sum_256(ss, part);
+        const float rinv = 1.0f / sqrtf(ss / (float)gs + a.eps);
+        for (int i = g * gs + tid(); i < (g + 1) * gs; i += 256)
+        {
+            const float hn = v[i] * rinv * ro_ld<T>((const T*)a.w_in + i);
+            float o = hn;
+            if (a.conv_w)
+            {
+                const T* cw = (const T*)a.conv_w + (long long)i * a.taps;
+                float acc = ro_ld<T>(cw + a.taps - 1) * hn;
+                float carry = hn;                                // walks the tail from its newest entry: entry j moves to j - 1
+                for (int j = a.taps - 2; j >= 0; j--)
+                {
+                    const float old = pos - (a.taps - 1 - j) >= 0 ? tl[(long long)j * a.width + i] : 0.0f;
+                    acc = fmaf(ro_ld<T>(cw + j), old, acc);
+                    tl[(long long)j * a.width + i] = carry;
+                    carry = old;
+                }
+                o = hn + acc;
+            }
+            if (a.out_f32) ((float*)a.out)[(long long)r * a.width + i] = o; else ro_st<T>((T*)a.out + (long long)r * a.width + i, o);
+        }
+    }
+}
+
+// ---- token embedding + hashed token-pair embedding + norm ------------------------------------------------------------------------
+// x = n_g(table[t] * scale + pair[(t' mul_prev + t mul_cur) mod buckets]) w, t' = the sequence's previous token: the row in front
+// when that belongs to the same sequence, else what the slot keeps (prev_tok int32 [slots]); row `buckets` of the pair table at
+// position 0.  fused (single-row spans): the slot takes the row's token here, otherwise token_state_kernel does after the launch.
+
+struct EmbedPairArgs
+{
+    const void* table; const void* pair; const void* w;         // pair, w nullable
+    const int* ids; int* prev_tok; const int* row_seq; const int* row_pos;
+    float* x;
+    int width, vocab, buckets, mul_prev, mul_cur, groups, fused; float scale, eps;
+};
+
+template <typename T>
+KERNEL void __launch_bounds__(256) embed_pair_kernel(const EmbedPairArgs a)
+{
+    DYN_SMEM(smem);
+    SHARED float part[4];
+    float* v = (float*)smem;
+    const int r = bid_x();
+    const int id = min(max(a.ids[r], 0), a.vocab - 1);
+    const int sq = a.row_seq[r], pos = a.row_pos[r];
+    long long prow = a.buckets;
+    if (a.pair && pos > 0)
+    {
+        const int pt = (!a.fused && r > 0 && a.row_seq[r - 1] == sq) ? a.ids[r - 1] : a.prev_tok[sq];
+        const long long hsh = ((long long)pt * a.mul_prev + (long long)id * a.mul_cur) % a.buckets;
+        prow = hsh < 0 ? hsh + a.buckets : hsh;
+    }
+    const T* src = (const T*)a.table + (long long)id * a.width;
+    const T* psrc = a.pair ? (const T*)a.pair + prow * a.width : nullptr;
+    float* xr = a.x + (long long)r * a.width;
+    for (int i = tid(); i < a.width; i += 256)
+    {
+        float t = ro_ld<T>(src + i) * a.scale;
+        if (psrc) t += ro_ld<T>(psrc + i);
+        v[i] = t;
+        if (!a.w) xr[i] = t;
+    }
+    if (a.w)
+    {
+        const int gs = a.width / a.groups;
+        for (int g = 0; g < a.groups; g++)
+        {
+            float ss = 0.0f;
+            for (int i = g * gs + tid(); i < (g + 1) * gs; i += 256) ss = fmaf(v[i], v[i], ss);
+            ss = block_sum_256(ss, part);
+            const float rinv = 1.0f / sqrtf(ss / (float)gs + a.eps);
+            for (int i = g * gs + tid(); i < (g + 1) * gs; i += 256) xr[i] = v[i] * rinv * ro_ld<T>((const T*)a.w + i);
+        }
+    }
+    else block_sync();
+    if (a.fused && tid() == 0) a.prev_tok[sq] = id;             // behind a barrier: every thread has read the slot
+}
+
+KERNEL void __launch_bounds__(64) token_state_kernel(const int* ids, int* prev_tok, const int* span_row0, const int* span_rows,
+                                                      const int* row_seq, int spans, int vocab)
+{
+    const int s = bid_x() * 64 + tid();
+    if (s >= spans) return;
+    const int last = span_row0[s] + span_rows[s] - 1;
+    prev_tok[row_seq[last]] = min(max(ids[last], 0), vocab - 1);
+}
+
 // ---- router -----------------------------------------------------------------------------------------------------------------
 // One wave per token.  logits fp32 [rows, n_total]; scores = softmax over all n_total; the `top` largest (score + correction) win
 // (first index on a tie); weight = score / (sum of the chosen scores + 1e-20) * scale.  sigmoid_scores: scores = sigmoid(logits),
@@ -606,6 +763,76 @@ extern "C" int exl2_span_last_rows(const float* src, int ld, float* slot_rows, i
     EXL2_REQUIRE(src && slot_rows && span_row0 && span_rows && row_seq && width > 0 && ld >= width, "span_last_rows: bad operand");
     if (spans <= 0) return EXL2_OK;
     LAUNCH(span_last_row_kernel, dim3(spans, (width + 255) / 256), dim3(256), 0, stream, src, ld, slot_rows, width, span_row0, span_rows, row_seq);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+extern "C" int exl2_sandwich_norm(float* x, const float* y, float ya, const float* y2, float yb, const float* moe_y, int top,
+                                  const void* w_out, float mult, const void* w_in, void* out, int out_f32, const int* row_idx,
+                                  const void* conv_w, float* tail, const int* row_seq, const int* row_pos, int taps, int dtype, int rows,
+                                  int width, int groups, float eps, void* stream)
+{
+    EXL2_REQUIRE(x, "sandwich_norm: null stream");
+    EXL2_REQUIRE(dtype == 0 || dtype == 1, "sandwich_norm: dtype must be 0 (bfloat16) or 1 (float32)");
+    const bool pending = y || y2 || moe_y;
+    EXL2_REQUIRE(!pending || w_out, "sandwich_norm: a sublayer's output needs the weight of the norm behind it");
+    EXL2_REQUIRE(!moe_y || top > 0, "sandwich_norm: expert outputs need their count per row");
+    EXL2_REQUIRE(pending || out, "sandwich_norm: neither an addition nor a norm");
+    EXL2_REQUIRE(!out || w_in, "sandwich_norm: an output needs the weight of the norm in front of it");
+    EXL2_REQUIRE(!(row_idx && (pending || conv_w)), "sandwich_norm: gathered rows take no addition and no convolution");
+    EXL2_REQUIRE(!conv_w || (out && taps >= 1 && (taps == 1 || (tail && row_seq && row_pos))), "sandwich_norm: the convolution needs an output, the slots' tails and the rows' places");
+    EXL2_REQUIRE(groups > 0 && width > 0 && width % groups == 0, "sandwich_norm: %d values in %d groups", width, groups);
+    EXL2_REQUIRE((size_t)width * 4 <= 160 * 1024 - 64, "sandwich_norm: row of %d values does not fit the LDS", width);
+    if (rows <= 0) return EXL2_OK;
+    SandwichArgs a;
+    a.x = x; a.y = y; a.ya = ya; a.y2 = y2; a.yb = yb; a.moe_y = moe_y; a.top = top; a.w_out = w_out; a.mult = mult; a.w_in = w_in;
+    a.out = out; a.out_f32 = out_f32 || dtype == 1; a.row_idx = row_idx; a.conv_w = conv_w; a.tail = tail; a.row_seq = row_seq;
+    a.row_pos = row_pos; a.taps = taps; a.width = width; a.groups = groups; a.eps = eps;
+    const size_t smem = (size_t)width * 4;
+    if (smem > 48 * 1024)
+    {
+        static bool attr_done[EXL2_MAX_DEVICES];
+        if (exl2_first_on_device(attr_done))
+        {
+            (void)hipFuncSetAttribute((const void*)sandwich_norm_kernel<u16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)sandwich_norm_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        }
+    }
+    if (dtype == 0) LAUNCH(sandwich_norm_kernel<u16>, dim3(rows), dim3(256), smem, stream, a);
+    else LAUNCH(sandwich_norm_kernel<float>, dim3(rows), dim3(256), smem, stream, a);
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+extern "C" int exl2_embed_pair(const void* table, const void* pair, const void* w, const int* ids, int* prev_tok, const int* row_seq,
+                               const int* row_pos, const int* span_row0, const int* span_rows, int spans, int max_span_rows, float* x,
+                               int dtype, int rows, int width, int vocab, int buckets, int mul_prev, int mul_cur, float scale, int groups,
+                               float eps, void* stream)
+{
+    EXL2_REQUIRE(table && ids && x && row_seq && row_pos, "embed_pair: null operand");
+    EXL2_REQUIRE(dtype == 0 || dtype == 1, "embed_pair: dtype must be 0 (bfloat16) or 1 (float32)");
+    EXL2_REQUIRE(!pair || (prev_tok && buckets > 0 && span_row0 && span_rows && spans > 0 && max_span_rows > 0),
+                 "embed_pair: the pair table needs its size, the slots' tokens and the step's spans");
+    EXL2_REQUIRE(width > 0 && vocab > 0 && (!w || (groups > 0 && width % groups == 0)), "embed_pair: bad shape");
+    EXL2_REQUIRE((size_t)width * 4 <= 160 * 1024 - 64, "embed_pair: row of %d values does not fit the LDS", width);
+    if (rows <= 0) return EXL2_OK;
+    EmbedPairArgs a;
+    a.table = table; a.pair = pair; a.w = w; a.ids = ids; a.prev_tok = prev_tok; a.row_seq = row_seq; a.row_pos = row_pos; a.x = x;
+    a.width = width; a.vocab = vocab; a.buckets = buckets; a.mul_prev = mul_prev; a.mul_cur = mul_cur; a.groups = groups > 0 ? groups : 1;
+    a.fused = pair && max_span_rows == 1; a.scale = scale; a.eps = eps;
+    const size_t smem = (size_t)width * 4;
+    if (smem > 48 * 1024)
+    {
+        static bool attr_done[EXL2_MAX_DEVICES];
+        if (exl2_first_on_device(attr_done))
+        {
+            (void)hipFuncSetAttribute((const void*)embed_pair_kernel<u16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)embed_pair_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        }
+    }
+    if (dtype == 0) LAUNCH(embed_pair_kernel<u16>, dim3(rows), dim3(256), smem, stream, a);
+    else LAUNCH(embed_pair_kernel<float>, dim3(rows), dim3(256), smem, stream, a);
+    if (pair && !a.fused) LAUNCH(token_state_kernel, dim3((spans + 63) / 64), dim3(64), 0, stream, ids, prev_tok, span_row0, span_rows, row_seq, spans, vocab);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;
 }

@@ -31,7 +31,9 @@ struct ConvArgs
 {
     const float* in; int ld;                 // [rows, ld]: the channels start at the pointer
     const void* w; const void* bias;         // [channels, taps], [channels]
-    float* out; int ldo;                     // [rows, ldo]
+    void* out; int ldo;                      // [rows, ldo] fp32, or the operand dtype (out_f32 == 0)
+    int out_f32;
+    int residual;                            // 0: out = silu(conv + bias);  1: out = in + conv + bias (no activation)
     float* tail;                             // [slots, taps - 1, channels]: inputs of the last taps - 1 positions of every sequence
     const int* span_row0; const int* span_rows; const int* row_seq; const int* row_pos;
     int channels, taps;
@@ -87,7 +89,9 @@ KERNEL void __launch_bounds__(256) conv_silu_kernel(const ConvArgs a)
             if (k == a.taps - 1) win[k] = xin[i];                // after the shift the newest value belongs at index taps - 1
             if (k < a.taps) acc = fmaf(w[k], win[k], acc);
         }
-        a.out[(long long)(r0 + t0 + i) * a.ldo + c] = ss_silu(acc);
+        const float o = a.residual ? xin[i] + acc : ss_silu(acc);
+        if (a.out_f32) ((float*)a.out)[(long long)(r0 + t0 + i) * a.ldo + c] = o;
+        else ss_st<T>((T*)a.out + (long long)(r0 + t0 + i) * a.ldo + c, o);
     }
     if (a.roll_tail && a.taps > 1)
     {
@@ -563,9 +567,23 @@ KERNEL void __launch_bounds__(256) gated_group_norm_kernel(const float* y, int l
 
 // ---- C ABI ----------------------------------------------------------------------------------------------------------------------
 
+extern "C" int exl2_conv_rows_ex(const float* in, int ld, const void* w, const void* bias, void* out, int ldo, int out_f32, int residual,
+                                 float* tail, const int* span_row0, const int* span_rows, int spans, int max_span_rows,
+                                 const int* row_seq, const int* row_pos, int dtype, int channels, int taps, void* stream);
+
 extern "C" int exl2_conv_silu_rows(const float* in, int ld, const void* w, const void* bias, float* out, int ldo, float* tail,
                                    const int* span_row0, const int* span_rows, int spans, int max_span_rows, const int* row_seq,
                                    const int* row_pos, int dtype, int channels, int taps, void* stream)
+{
+    return exl2_conv_rows_ex(in, ld, w, bias, out, ldo, 1, 0, tail, span_row0, span_rows, spans, max_span_rows, row_seq, row_pos, dtype,
+                             channels, taps, stream);
+}
+
+/* The same convolution with a choice of output: residual = 0: silu(conv + bias); 1: in + conv + bias, no activation (what a
+   sublayer reads when its input passes a short convolution beside the identity).  out fp32, or the operand dtype with out_f32 = 0. */
+extern "C" int exl2_conv_rows_ex(const float* in, int ld, const void* w, const void* bias, void* out, int ldo, int out_f32, int residual,
+                                 float* tail, const int* span_row0, const int* span_rows, int spans, int max_span_rows,
+                                 const int* row_seq, const int* row_pos, int dtype, int channels, int taps, void* stream)
 {
     EXL2_REQUIRE(in && w && out && tail && span_row0 && span_rows && row_seq && row_pos, "conv_silu_rows: null operand");
     EXL2_REQUIRE(dtype == 0 || dtype == 1, "conv_silu_rows: dtype must be 0 (bfloat16) or 1 (float32)");
@@ -575,6 +593,7 @@ extern "C" int exl2_conv_silu_rows(const float* in, int ld, const void* w, const
     ConvArgs a;
     a.in = in; a.ld = ld; a.w = w; a.bias = bias; a.out = out; a.ldo = ldo; a.tail = tail; a.span_row0 = span_row0; a.span_rows = span_rows;
     a.row_seq = row_seq; a.row_pos = row_pos; a.channels = channels; a.taps = taps;
+    a.out_f32 = out_f32 || dtype == 1; a.residual = residual;
     a.roll_tail = max_span_rows <= CONV_TOKENS;
     const dim3 grid((channels + 255) / 256, (max_span_rows + CONV_TOKENS - 1) / CONV_TOKENS, spans);
     if (dtype == 0)

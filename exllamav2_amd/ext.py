@@ -779,6 +779,7 @@ class ExtC:
 
     EPI_NONE, EPI_MUL_SIGMOID_AUX, EPI_SILU_AUX_MUL, EPI_CLAMPED_GLU, EPI_RELU_SQUARED, EPI_SOFT_CAP = 0, 1, 2, 3, 4, 5
     EPI_SCALE, EPI_TANH, EPI_ROW_SCALED_RELU_SQUARED = 6, 7, 8        # acc * limit; tanh(acc); relu(aux[row] * acc)^2
+    EPI_ROW_SCALED_SILU_SCALED, EPI_AUX_MUL = 9, 10                   # silu(aux[row] * acc) * aux[row]; acc * aux
 
     @staticmethod
     def _dense_code(dtype) -> int:
@@ -1069,6 +1070,71 @@ class ExtC:
             self._ptr(nrows, torch.int32, "span_rows"), self._ptr(chunk0, torch.int32, "span_chunk0"), int(n), int(chunk), int(total),
             self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"), self._ptr(zbuf, torch.float32, "zbuf"),
             self._ptr(dbuf, torch.float32, "dbuf"), int(heads), int(n_key), int(n_val), float(eps), self._stream(out)))
+
+    # ---- sandwich-normed residual step, token-pair embedding (csrc/rowops.hip), convolution variants (csrc/ssm.hip), matrix-state
+    # recurrences (csrc/gated_scan.hip) ------------------------------------------------------------------------------------------
+
+    def sandwich_norm(self, x32, w_out, mult: float, w_in, out, rows: int, groups: int, eps: float, y=None, ya: float = 1.0, y2=None,
+                      yb: float = 1.0, moe_y=None, top: int = 0, row_idx=None, conv_w=None, tail=None, row_seq=None, row_pos=None,
+                      taps: int = 0, dtype=None) -> None:
+        """x32 += mult * n_g(ya y + yb y2 + expert rows) w_out (when any of them is given), then out = n_g(x32) w_in (out may be None);
+        conv_w + tail + row_seq + row_pos: single-row spans read out through the short convolution over the slot's last normed rows"""
+        width = x32.shape[-1]
+        wt = w_in if w_in is not None else w_out
+        dt = dtype if dtype is not None else wt.dtype
+        self.lib.check(self.lib.exl2_sandwich_norm(
+            self._ptr(x32, torch.float32, "x32"), self._ptr(y, torch.float32, "y"), float(ya), self._ptr(y2, torch.float32, "y2"), float(yb),
+            self._ptr(moe_y, torch.float32, "moe_y"), int(top), self._ptr(w_out, dt, "w_out"), float(mult), self._ptr(w_in, dt, "w_in"),
+            self._ptr(out, None, "out"), int(out is not None and out.dtype is torch.float32), self._ptr(row_idx, torch.int32, "row_idx"),
+            self._ptr(conv_w, dt, "conv_w"), self._ptr(tail, torch.float32, "tail"), self._ptr(row_seq, torch.int32, "row_seq"),
+            self._ptr(row_pos, torch.int32, "row_pos"), int(taps), self._dense_code(dt), int(rows), int(width), int(groups), float(eps),
+            self._stream(x32)))
+
+    def embed_pair(self, table, pair, w, ids, prev_tok, row_seq, row_pos, spans, x32, buckets: int, mul_prev: int, mul_cur: int,
+                   scale: float, groups: int, eps: float) -> None:
+        """x32 = n_g(table[ids] * scale + pair[hash(previous token, token)]) w; spans = (span_row0, span_rows, n, longest span)"""
+        row0, nrows, n, longest = spans
+        rows, width = ids.numel(), table.shape[1]
+        self.lib.check(self.lib.exl2_embed_pair(
+            self._ptr(table, None, "table"), self._ptr(pair, table.dtype, "pair"), self._ptr(w, table.dtype, "w"),
+            self._ptr(ids, torch.int32, "ids"), self._ptr(prev_tok, torch.int32, "prev_tok"), self._ptr(row_seq, torch.int32, "row_seq"),
+            self._ptr(row_pos, torch.int32, "row_pos"), self._ptr(row0, torch.int32, "span_row0"), self._ptr(nrows, torch.int32, "span_rows"),
+            int(n), int(longest), self._ptr(x32, torch.float32, "x32"), self._dense_code(table.dtype), int(rows), int(width),
+            table.shape[0], int(buckets), int(mul_prev), int(mul_cur), float(scale), int(groups), float(eps), self._stream(x32)))
+
+    def conv_rows(self, f, ld: int, f_off: int, w, bias, out, tail, spans, row_seq, row_pos, channels: int, taps: int,
+                  residual: bool = False) -> None:
+        """conv_silu_rows with a choice of output: residual -> out = in + conv (+ bias), no activation; out fp32 or w's dtype"""
+        row0, nrows, n, longest = spans
+        self.lib.check(self.lib.exl2_conv_rows_ex(
+            self._ptr(f, torch.float32, "f") + f_off * 4, int(ld), self._ptr(w, None, "w"), self._ptr(bias, w.dtype, "bias"),
+            self._ptr(out, None, "out"), out.shape[-1], int(out.dtype is torch.float32), int(residual), self._ptr(tail, torch.float32, "tail"),
+            self._ptr(row0, torch.int32, "span_row0"), self._ptr(nrows, torch.int32, "span_rows"), int(n), int(longest),
+            self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"), self._dense_code(w.dtype), int(channels),
+            int(taps), self._stream(out)))
+
+    SCAN_FORGET_WRITES, SCAN_DELTA = 0, 1
+
+    def gated_scan(self, mode: int, f, ld: int, q_off: int, k_off: int, v, ldv: int, v_off: int, norm_w, out, state, spans, row_seq, row_pos,
+                   heads: int, qk_heads: int, n_key: int, n_val: int, eps: float, q_scale: float = 1.0, lower=None, gate_off: int | None = None,
+                   beta_off: int = 0, dt_off: int = 0, dt_bias=None, a_log=None, qk=None, ldqk: int = 0) -> None:
+        """f fp32 [rows, ld]: the mixer's projections -- mode 0: q pre-activation at q_off, forget-gate pre-activation at k_off; mode 1:
+        beta / decay inputs / output gate at beta_off / dt_off / gate_off, q and k in `qk` fp32 [rows, ldqk] at q_off / k_off (the
+        convolved rows).  v fp32 [rows, ldv] at v_off.  out [rows, heads * n_val] operand dtype or fp32."""
+        row0, nrows, n, _longest = spans
+        pf = self._ptr(f, torch.float32, "f")
+        pqk = self._ptr(qk, torch.float32, "qk") if qk is not None else pf
+        lqk = int(ldqk) if qk is not None else int(ld)
+        delta = mode == self.SCAN_DELTA
+        self.lib.check(self.lib.exl2_gated_scan(
+            int(mode), pqk + q_off * 4, lqk, pqk + k_off * 4, lqk, self._ptr(v, torch.float32, "v") + v_off * 4, int(ldv),
+            (pf + gate_off * 4) if gate_off is not None else None, int(ld), (pf + beta_off * 4) if delta else None, int(ld),
+            (pf + dt_off * 4) if delta else None, int(ld), self._ptr(dt_bias, torch.float32, "dt_bias"),
+            self._ptr(a_log, torch.float32, "a_log"), self._ptr(lower, torch.float32, "lower"), self._ptr(norm_w, torch.float32, "norm_w"),
+            self._ptr(out, None, "out"), out.shape[-1], int(out.dtype is torch.float32), self._ptr(state, torch.float32, "state"),
+            self._ptr(row0, torch.int32, "span_row0"), self._ptr(nrows, torch.int32, "span_rows"), int(n),
+            self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"), int(heads), int(qk_heads), int(n_key),
+            int(n_val), float(q_scale), float(eps), self._stream(out)))
 
     def graph_begin_capture(self, stream: int | None) -> None:
         self.lib.check(self.lib.exl2_graph_begin_capture(stream))

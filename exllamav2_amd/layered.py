@@ -2,8 +2,10 @@
 registries, on an fp32 residual stream.  The residual style is the configuration's: post-norm steps
 x <- norm(alpha x + sublayer(x)) (1 + w)  (RMS norm, a `head` matrix), or pre-norm steps  x <- x + sublayer(layer_norm(x))  (weight and
 bias, logits from the embedding table, optional soft cap), or pre-norm steps with scalar-gain RMS norms and a token shift in front
-of every mixer (a `head` matrix, scaled logits).  Mixers: latent attention, windowed / chunked attention (pooled blocks, sinks, shared
-keys and values), state-space scan, decaying linear attention; a stack may mix them -- each keeps what it needs between steps (pages
+of every mixer (a `head` matrix, scaled logits), or sandwich-normed steps  x <- x + mult n_g(sublayer(conv_in(n_g(x) w))) w'  with
+grouped RMS norms, a short input convolution and a token-pair table beside the embedding.  Mixers: latent attention, windowed /
+chunked / plain causal attention (pooled blocks, sinks, shared keys and values), state-space scan, decaying linear attention, linear
+attention whose forget gate writes, gated delta rule, two mixers side by side; a stack may mix them -- each keeps what it needs between steps (pages
 of keys and values, per-slot recurrent state) under one page pool.
 
 The model has ONE forward, `step(batch, cache)`: the rows of a step are a flat list of tokens, each with its sequence slot and
@@ -21,9 +23,11 @@ from .config import LayeredConfig
 from .dense_linear import DenseLinear
 from .ext import ext_c
 from .latent_attn import LatentAttention
+from .linear_attn import ForgetGateLinearAttention, GatedDeltaRule
 from .mlp import DenseActMLP, DenseGatedMLP
 from .moe_mlp import ScoredMoEMLP, SigmoidMoEMLP
-from .rmsnorm import PostNorm, PreLayerNorm, PreShiftRMSNorm
+from .parallel_mixer import ParallelMixer
+from .rmsnorm import PostNorm, PreLayerNorm, PreShiftRMSNorm, SandwichNorm
 from .ssm import StateSpaceMixer
 from .window_attn import WindowAttention
 from .wkv import DecayLinearAttention
@@ -62,6 +66,37 @@ def _state_space(model, key, idx, spec):
                            groups=int(m.get("groups", 1)), norm_groups=int(m.get("norm_groups", 1)), taps=int(m["conv"]))
 
 
+def _causal_attention(model, key, idx, m, out_tag="mix.y"):
+    """plain causal softmax attention: every earlier token is visible, no sink, no gate, values as they are"""
+    rot = m.get("rot") or {}
+    return WindowAttention(model, key, idx, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads") or m["heads"]), dim=int(m["dim"]),
+                           vdim=int(m.get("vdim") or m["dim"]), window=1 << 30, pool=0, rot_base=float(rot.get("base", 10000.0)),
+                           rot_dims=int(rot.get("dims", 0)), rot_scaling=rot.get("scaling"), scale=float(m["scale"]), rotate_values=False,
+                           out_tag=out_tag)
+
+
+def _parallel(model, key, idx, spec):
+    """softmax attention (left) beside a state-space scan (right) on the same input"""
+    m = spec["mixer"]
+    r = m["right"]
+    left = _causal_attention(model, key + ".left", (idx, "left"), m["left"], out_tag="mix.y.left")
+    right = StateSpaceMixer(model, key + ".right", (idx, "right"), heads=int(r["heads"]), vdim=int(r["vdim"]), state=int(r["state"]),
+                            groups=int(r.get("groups", 1)), norm_groups=int(r.get("norm_groups", 1)), taps=int(r["conv"]),
+                            out_tag="mix.y.right")
+    return ParallelMixer(model, key, idx, left, right, float(m.get("left_scale", 1.0)), float(m.get("right_scale", 1.0)))
+
+
+def _forget_gate_attention(model, key, idx, spec):
+    m = spec["mixer"]
+    return ForgetGateLinearAttention(model, key, idx, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]))
+
+
+def _delta_rule(model, key, idx, spec):
+    m = spec["mixer"]
+    return GatedDeltaRule(model, key, idx, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads") or m["heads"]), dim=int(m["dim"]),
+                          vdim=int(m["vdim"]), taps=int(m["conv"]))
+
+
 def _dense_mlp(model, key, idx, spec):
     if model.config.residual == "pre_ln":                      # two matrices, squared relu between them
         return DenseActMLP(model, key, idx)
@@ -70,16 +105,18 @@ def _dense_mlp(model, key, idx, spec):
 
 def _moe_mlp(model, key, idx, spec):
     r, e = spec["router"], spec["expert"]
-    if model.config.residual == "pre_rms_shift":              # sigmoid scores weigh the experts' inputs; a shared expert beside them
+    if model.config.residual in ("pre_rms_shift", "sandwich"):        # sigmoid scores weigh the experts' inputs; a shared expert beside them
         shared = spec.get("shared")
         return SigmoidMoEMLP(model, key, idx, experts=int(r["experts"]), top=int(r["top"]), ff=int(e["ff"]),
-                             shared_ff=(int(shared["ff"]) if shared else None), route_scale=float(r.get("scale", 1.0)))
+                             shared_ff=(int(shared["ff"]) if shared else None), route_scale=float(r.get("scale", 1.0)),
+                             act="silu_glu" if model.config.residual == "sandwich" else "relu2")
     return ScoredMoEMLP(model, key, idx, experts=int(r["experts"]), identity=int(r.get("identity", 0)), top=int(r["top"]),
                         route_scale=float(r["scale"]), ff=int(e["ff"]), limit=float(e["limit"]))
 
 
 # config `type` -> builder(model, key, layer index, layer spec)
-MIXERS = {"latent_attention": _latent_attention, "attention": _window_attention, "mamba2": _state_space, "wkv": _decay_linear_attention}
+MIXERS = {"latent_attention": _latent_attention, "attention": _window_attention, "mamba2": _state_space, "wkv": _decay_linear_attention,
+          "parallel": _parallel, "hgrn2": _forget_gate_attention, "delta": _delta_rule}
 FEED_FORWARDS = {"dense": _dense_mlp, "moe": _moe_mlp}       # config `mlp.kind` -> builder(model, key, layer index, mlp spec)
 
 
@@ -161,9 +198,15 @@ class LayeredModel:
         self.embed = need("embed")
         if tuple(self.embed.shape) != (cfg.vocab, cfg.width):
             raise RuntimeError(f"embed is {tuple(self.embed.shape)}, config says {(cfg.vocab, cfg.width)}")
-        pre = cfg.residual in ("pre_ln", "pre_rms_shift")
+        pre = cfg.residual in ("pre_ln", "pre_rms_shift", "sandwich")
 
         def make_norm(name, shift=None):
+            if cfg.residual == "sandwich":
+                # `<layer>.norm1` / `.norm2` in front of a sublayer, `.norm1b` / `.norm2b` behind it, `.canon1` / `.canon2` its input convolution
+                inner = name != "final.norm"
+                conv = need(name.replace("norm", "canon"), optional=cfg.input_conv_taps <= 0) if inner else None
+                return SandwichNorm(self.ext, name, need(name), need(name + "b") if inner else None, conv,
+                                    cfg.norm_groups, cfg.norm_eps, cfg.residual_mult)
             if cfg.residual == "pre_rms_shift":
                 return PreShiftRMSNorm(self.ext, name, need(name), cfg.norm_eps, shift=need(shift) if shift else None)
             if pre:
@@ -208,6 +251,13 @@ class LayeredModel:
                     self.sublayers.append((norm2, ff, False, i))
         else:
             self.final_norm = need("final.norm")
+        self.pair_table = self.embed_norm = None
+        if cfg.residual == "sandwich":
+            self.embed_norm = need("embed.norm")
+            if cfg.pair_embedding is not None:
+                self.pair_table = need("bigram")
+                if tuple(self.pair_table.shape) != (cfg.pair_embedding["buckets"] + 1, cfg.width):
+                    raise RuntimeError(f"bigram is {tuple(self.pair_table.shape)}, config says {(cfg.pair_embedding['buckets'] + 1, cfg.width)}")
         self.head = DenseLinear(self.ext, "head", self.embed if cfg.tied_head else need("head"))
         self.loaded = True
         return self
@@ -222,10 +272,20 @@ class LayeredModel:
     # ---- cache ----------------------------------------------------------------------------------------------------------------
 
     def make_cache(self, pool: PagePool):
-        if any(hasattr(mixer, "make_state") for mixer, *_rest in self.layers):
+        if any(hasattr(mixer, "make_state") or hasattr(mixer, "make_states") for mixer, *_rest in self.layers):
             norm_states = {i: norm1.make_state(pool, self.width) for i, (_m, norm1, *_r) in enumerate(self.layers) if hasattr(norm1, "make_state")}
-            return LayerStates(pool, {i: mixer.make_state(pool, self.dtype) for i, (mixer, *_rest) in enumerate(self.layers)},
-                               norm_states=norm_states)
+            norm_states.update({(i, "ff"): norm2.make_state(pool, self.width) for i, (_m, _n1, _ff, norm2) in enumerate(self.layers)
+                                if norm2 is not None and hasattr(norm2, "make_state")})
+            if getattr(self, "pair_table", None) is not None:
+                from .cache import SlotState
+                norm_states["embed"] = SlotState(pool, {"prev_token": ()}, dtype=torch.int32)
+            per_layer = {}
+            for i, (mixer, *_rest) in enumerate(self.layers):
+                if hasattr(mixer, "make_states"):                 # several states under keys of the mixer's own ((layer, "left"), ...)
+                    per_layer.update(mixer.make_states(pool, self.dtype))
+                else:
+                    per_layer[i] = mixer.make_state(pool, self.dtype)
+            return LayerStates(pool, per_layer, norm_states=norm_states)
         widths, owner = {}, {}
         for i, (mixer, *_rest) in enumerate(self.layers):
             if mixer.kv_from is None:
@@ -245,6 +305,8 @@ class LayeredModel:
             return self._step_pre_norm(batch, cache)
         if cfg.residual == "pre_rms_shift":
             return self._step_pre_rms_shift(batch, cache)
+        if cfg.residual == "sandwich":
+            return self._step_sandwich(batch, cache)
         x32 = self.buf("x32", (rows, self.width), torch.float32)
         xh = x32 if self.dtype is torch.float32 else self.buf("xh", (rows, self.width), self.dtype)
         ext.embed_scale(self.embed, batch.ids, x32, xh, cfg.embedding_scale)
@@ -318,3 +380,38 @@ class LayeredModel:
         scaled = cfg.logit_scale != 1.0
         return self.head.forward(xn, batch.n_logits, out=self.buf("logits", (batch.n_logits, self.vocab), f32),
                                  epi=ext.EPI_SCALE if scaled else ext.EPI_NONE, limit=cfg.logit_scale)
+
+    def _step_sandwich(self, batch: StepBatch, cache) -> torch.Tensor | None:
+        """x <- x + mult n_g(mixer(conv_in(n_g(x) w1))) w1b, x <- x + mult n_g(ff(conv_in(n_g(x) w2))) w2b: what lies between two
+        sublayers -- the norm behind the first (over a linear's output, the weighted results of two mixers side by side, or a shared
+        expert's output plus the chosen experts' rows), the residual addition, the norm in front of the second and, in steps of single
+        tokens, its input convolution -- is one launch.  The embedding adds a row of the token-pair table chosen by the previous and the
+        current token (the previous token is kept per slot) and is normed.  Logits: head(n_g(x) w) for the wanted rows."""
+        ext, cfg, rows, f32 = self.ext, self.config, batch.rows, torch.float32
+        x32 = self.buf("x32", (rows, self.width), f32)
+        xh = self.buf("xh", (rows, self.width), self.dtype)
+        pe = cfg.pair_embedding or {"buckets": 0, "mul_prev": 0, "mul_cur": 0}
+        est = cache.norm_state("embed")
+        ext.embed_pair(self.embed, self.pair_table, self.embed_norm, batch.ids, est["prev_token"] if est is not None else None, batch.row_seq,
+                       batch.row_pos, batch.spans_dev, x32, pe["buckets"], pe["mul_prev"], pe["mul_cur"], cfg.embedding_scale,
+                       cfg.norm_groups, cfg.norm_eps)
+        pending = None
+        for norm, module, is_mixer, layer in self.sublayers:
+            norm.forward(x32, pending, xh, rows, model=self, batch=batch, state=cache.norm_state(layer if is_mixer else (layer, "ff")),
+                         dtype=self.dtype)
+            if is_mixer:
+                y = module.forward(xh, rows, batch, cache)
+                pending = (norm,) + (tuple(y) if isinstance(y, tuple) else (y, 1.0, None, 1.0)) + (None, 0)
+            else:
+                y, mix = module.forward(xh, rows)
+                pending = (norm, y, 1.0, None, 1.0) + ((mix[0], mix[1].shape[-1]) if mix is not None else (None, 0))
+        xn = self.buf("xn", (max(batch.n_logits, 1), self.width), self.dtype)
+        if batch.logits_all_rows and batch.n_logits == rows:
+            self.final_norm.forward(x32, pending, xn, rows, dtype=self.dtype)       # the last addition and the final norm in one launch
+        else:
+            if pending is not None:
+                self.final_norm.forward(x32, pending, None, rows, dtype=self.dtype)
+            if batch.n_logits == 0:
+                return None
+            self.final_norm.forward(x32, None, xn, batch.n_logits, row_idx=batch.logit_rows, dtype=self.dtype)
+        return self.head.forward(xn, batch.n_logits, out=self.buf("logits", (batch.n_logits, self.vocab), f32))

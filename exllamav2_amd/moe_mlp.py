@@ -127,21 +127,27 @@ class SigmoidMoEMLP:
     sum_e expert_e(s_e h), expert(z) = W_down act(W_up z) with act = relu^2 and no gate matrix; since W_up (s h) = s (W_up h) the
     up projection runs on h and the weight enters in its epilogue, in front of the activation (csrc/dense.hip).  A shared expert of
     the same form (its own width) runs for every token: as wide as the routed ones it is stacked behind them and rides their
-    launches as one more pair per token, otherwise it runs as a two-matrix feed-forward of its own.  Few rows: every (token, choice) pair names its expert's slab; many rows:
+    launches as one more pair per token, otherwise it runs as a feed-forward of its own.  `act="silu_glu"`: experts are gated units
+    W_down (silu(W_gate z) * W_up z); with z = s h the gate launch leaves silu(s g) s and the up launch multiplies by it, so both
+    matrices still run on h.  Few rows: every (token, choice) pair names its expert's slab; many rows:
     one grouped launch per projection.  forward returns (y | None, mixture): y is the shared expert's output, the chosen experts'
     rows are added by the residual step's launch (rmsnorm.PreShiftRMSNorm)."""
 
     PAIR_ROWS_MAX = 64
 
-    def __init__(self, model, key: str, layer_idx: int, *, experts: int, top: int, ff: int, shared_ff: int | None, route_scale: float = 1.0):
+    def __init__(self, model, key: str, layer_idx: int, *, experts: int, top: int, ff: int, shared_ff: int | None, route_scale: float = 1.0,
+                 act: str = "relu2"):
         self.model, self.ext, self.key, self.layer_idx = model, model.ext, key, layer_idx
         self.experts, self.top, self.ff, self.shared_ff, self.route_scale = experts, top, ff, shared_ff, route_scale
+        self.glu = act == "silu_glu"
         if not 0 < top <= experts:
             raise ValueError(f"{key}: top {top} of {experts} experts")
+        if act not in ("relu2", "silu_glu"):
+            raise ValueError(f"{key}: unknown expert form '{act}'")
 
     def load(self, get):
         from .dense_linear import DenseLinear
-        from .mlp import DenseActMLP
+        from .mlp import DenseActMLP, DenseGatedMLP
         E, width = self.experts, self.model.width
         self.router = DenseLinear(self.ext, self.key + ".router", get("router"))
         # a shared expert as wide as the routed ones is stacked behind them as expert E: the router's launch names it for every token
@@ -151,19 +157,23 @@ class SigmoidMoEMLP:
         stack = lambda name: torch.stack([get(f"{n}.{name}") for n in names], 0)
         self.up = DenseLinear(self.ext, self.key + ".up", stack("up"))
         self.down = DenseLinear(self.ext, self.key + ".down", stack("down"))
+        self.gate = DenseLinear(self.ext, self.key + ".gate", stack("gate")) if self.glu else None
         self.slabs = len(names)
         if tuple(self.router.weight.shape) != (E, width) or tuple(self.up.weight.shape) != (self.slabs, self.ff, width) \
-                or tuple(self.down.weight.shape) != (self.slabs, width, self.ff):
+                or tuple(self.down.weight.shape) != (self.slabs, width, self.ff) \
+                or (self.glu and tuple(self.gate.weight.shape) != (self.slabs, self.ff, width)):
             raise RuntimeError(f"{self.key}: tensor shapes do not match the feed-forward's sizes")
         self.shared = None
         if self.shared_ff and not self.merged:
-            self.shared = DenseActMLP(self.model, self.key + ".shared", self.layer_idx).load(lambda n: get("shared." + n))
+            form = DenseGatedMLP if self.glu else DenseActMLP
+            self.shared = form(self.model, self.key + ".shared", self.layer_idx).load(lambda n: get("shared." + n))
             if self.shared.up.out_features != self.shared_ff:
                 raise RuntimeError(f"{self.key}: the shared expert is {self.shared.up.out_features} wide, config says {self.shared_ff}")
         return self
 
     def weight_bytes(self) -> int:
-        n = self.router.weight_bytes() + (self.up.weight_bytes() + self.down.weight_bytes()) // self.slabs * (self.top + int(self.merged))
+        per_slab = (self.up.weight_bytes() + self.down.weight_bytes() + (self.gate.weight_bytes() if self.glu else 0)) // self.slabs
+        n = self.router.weight_bytes() + per_slab * (self.top + int(self.merged))
         return n + (self.shared.weight_bytes() if self.shared is not None else 0)
 
     def forward(self, xh: torch.Tensor, rows: int):
@@ -182,8 +192,15 @@ class SigmoidMoEMLP:
         a = m.buf("moe.a", (pairs, ff), dt)
         y = m.buf("moe.y", (pairs, width), torch.float32)
         kw = dict(batch=S, groups=groups) if grouped else dict(w_sel=ids.view(-1), n_sel=S)
-        ext.dense_linear(xh, self.up.weight, a, pairs, ff, width, width, width, ff, swb=ff * width, x_div=per_row,
-                         aux=wts, ldaux=1, epi=ext.EPI_ROW_SCALED_RELU_SQUARED, **kw)
+        if self.glu:
+            g = m.buf("moe.g", (pairs, ff), torch.float32)
+            ext.dense_linear(xh, self.gate.weight, g, pairs, ff, width, width, width, ff, swb=ff * width, x_div=per_row,
+                             aux=wts, ldaux=1, epi=ext.EPI_ROW_SCALED_SILU_SCALED, **kw)
+            ext.dense_linear(xh, self.up.weight, a, pairs, ff, width, width, width, ff, swb=ff * width, x_div=per_row,
+                             aux=g, ldaux=ff, epi=ext.EPI_AUX_MUL, **kw)
+        else:
+            ext.dense_linear(xh, self.up.weight, a, pairs, ff, width, width, width, ff, swb=ff * width, x_div=per_row,
+                             aux=wts, ldaux=1, epi=ext.EPI_ROW_SCALED_RELU_SQUARED, **kw)
         ext.dense_linear(a, self.down.weight, y, pairs, width, ff, ff, ff, width, swb=width * ff, **kw)
         ys = self.shared.forward(xh, rows)[0] if self.shared is not None else None
         return ys, (y, ids, wts, S)

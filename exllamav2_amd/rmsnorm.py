@@ -79,3 +79,61 @@ class PreShiftRMSNorm:
         if self.shift is not None and out is not None:
             kw = dict(shift=self.shift, prev=state["prev"], hn=hn, row_seq=batch.row_seq, row_pos=batch.row_pos, spans=batch.spans_dev)
         self.ext.add_rms_shift(x32, y, out, rows, self.gain, self.eps, moe_y=moe_y, top=top, row_idx=row_idx, dtype=dtype, **kw)
+
+
+class SandwichNorm:
+    """The two norms around one sublayer of a sandwich-normed layer, x <- x + mult * n_g(f(conv_in(n_g(x) w_in))) w_out, where n_g is
+    an RMS norm taken separately over `groups` equal runs of the row and conv_in(a) = a + a short causal convolution of a over the
+    sequence (weights [width, taps], optional).  `forward` runs what lies BETWEEN two sublayers as one launch (csrc/rowops.hip:
+    sandwich_norm_kernel): the norm behind the previous sublayer (`pending`: its outputs and its SandwichNorm), the residual
+    addition, and this sublayer's norm in front.  The convolution's history is per-sequence state: `make_state` asks the pool for
+    the last taps - 1 normed rows per slot; steps of single tokens convolve and roll it inside the norm's launch, steps with longer
+    spans write the normed rows in fp32 and convolve in a second launch (csrc/ssm.hip: conv_silu_kernel in its residual form)."""
+
+    def __init__(self, ext, key: str, w_in: torch.Tensor, w_out: torch.Tensor | None, conv_w: torch.Tensor | None, groups: int, eps: float,
+                 mult: float):
+        self.ext, self.key, self.groups, self.eps, self.mult = ext, key, int(groups), float(eps), float(mult)
+        self.w_in = w_in.contiguous()
+        self.w_out = w_out.contiguous() if w_out is not None else None
+        self.conv_w = conv_w.contiguous() if conv_w is not None else None
+        width = self.w_in.numel()
+        if width % self.groups or (self.w_out is not None and self.w_out.numel() != width):
+            raise RuntimeError(f"{key}: {width} values in {groups} groups")
+        self.taps = 0
+        if self.conv_w is not None:
+            if self.conv_w.dim() != 2 or self.conv_w.shape[0] != width:
+                raise RuntimeError(f"{key}: the input convolution's weights are {tuple(self.conv_w.shape)}, the rows {width} wide")
+            self.taps = int(self.conv_w.shape[1])
+
+    def make_state(self, pool, width: int):
+        from .cache import SlotState
+        return SlotState(pool, {"tail": (max(self.taps - 1, 1), width)}) if self.taps > 1 else None
+
+    @staticmethod
+    def _pending_args(pending) -> dict:
+        """pending: None or (the sublayer's SandwichNorm, y | None, ya, y2 | None, yb, expert rows | None, rows per token)"""
+        if pending is None:
+            return dict(w_out=None, mult=0.0)
+        norm, y, ya, y2, yb, moe_y, top = pending
+        return dict(w_out=norm.w_out, mult=norm.mult, y=y, ya=ya, y2=y2, yb=yb, moe_y=moe_y, top=top)
+
+    def forward(self, x32: torch.Tensor, pending, out: torch.Tensor | None, rows: int, model=None, batch=None, state=None, row_idx=None,
+                dtype=None) -> None:
+        """out (operand dtype or fp32, [rows, width]) takes what this norm's sublayer reads; None: only the pending addition"""
+        ext, pa = self.ext, self._pending_args(pending)
+        w_out, mult = pa.pop("w_out"), pa.pop("mult")
+        if out is None:
+            ext.sandwich_norm(x32, w_out, mult, None, None, rows, self.groups, self.eps, dtype=dtype, **pa)
+        elif self.conv_w is None or row_idx is not None:
+            ext.sandwich_norm(x32, w_out, mult, self.w_in, out, rows, self.groups, self.eps, row_idx=row_idx, dtype=dtype, **pa)
+        elif self.taps == 1 or batch.spans_dev[3] == 1:
+            # no history needed, or single-token spans: norm, convolution and the roll of the slot's tail in one launch
+            ext.sandwich_norm(x32, w_out, mult, self.w_in, out, rows, self.groups, self.eps, conv_w=self.conv_w,
+                              tail=state["tail"] if state is not None else None, row_seq=batch.row_seq, row_pos=batch.row_pos,
+                              taps=self.taps, dtype=dtype, **pa)
+        else:
+            width = x32.shape[-1]
+            hn = model.buf("hn", (rows, width), torch.float32)
+            ext.sandwich_norm(x32, w_out, mult, self.w_in, hn, rows, self.groups, self.eps, dtype=dtype, **pa)
+            ext.conv_rows(hn, width, 0, self.conv_w, None, out, state["tail"], batch.spans_dev, batch.row_seq, batch.row_pos, width,
+                          self.taps, residual=True)

@@ -19,7 +19,8 @@ from .dense_linear import DenseLinear
 class StateSpaceMixer:
     CHUNKED_FROM = 8                                          # longest span of a step from which the chunked scan is taken
 
-    def __init__(self, model, key: str, layer_idx: int, *, heads: int, vdim: int, state: int, groups: int, norm_groups: int, taps: int):
+    def __init__(self, model, key: str, layer_idx: int, *, heads: int, vdim: int, state: int, groups: int, norm_groups: int, taps: int,
+                 out_tag: str = "mix.y"):
         self.model, self.ext, self.key, self.layer_idx = model, model.ext, key, layer_idx
         self.heads, self.vdim, self.state, self.groups, self.norm_groups, self.taps = heads, vdim, state, groups, norm_groups, taps
         self.inner = heads * vdim
@@ -27,6 +28,7 @@ class StateSpaceMixer:
         if heads % groups or self.inner % norm_groups:
             raise ValueError(f"{key}: {heads} heads in {groups} groups, {self.inner} values in {norm_groups} norm groups")
         self.kv_from = None
+        self.out_tag = out_tag                                    # scratch buffer of the result (a layer may run two mixers side by side)
         self.chunked_ok = self.ext.ssm_scan_chunked_supported(state, vdim) and self.inner % 4 == 0 and self.channels % 4 == 0
 
     def load(self, get):
@@ -74,4 +76,4 @@ class StateSpaceMixer:
             ext.ssm_scan(*scan_args, batch.row_seq, batch.row_pos, self.heads, self.groups, self.state, self.vdim)
         g = m.buf("ssm.g", (rows, inner), m.dtype)
         ext.gated_group_norm(y, f, self.n_front, self.norm_w, g, rows, inner, self.norm_groups, m.norm_eps)
-        return self.o.forward(g, rows, out=m.buf("mix.y", (rows, m.width), f32))
+        return self.o.forward(g, rows, out=m.buf(self.out_tag, (rows, m.width), f32))

@@ -15,8 +15,10 @@ pair layout, score scale, and the variants
     softcap      s_j <- softcap * tanh(s_j / softcap)
     sink_one     the denominator holds a constant 1 (a sink of score 0) instead of a learned exp(sink_i)
     kv_from      the layer has no key / value projections: it attends over the rows layer `kv_from` cached, with its own queries
-biases, per-head temperature and the learned sink are used when the checkpoint has them; a gate tensor of one row per head gates
-whole heads, one of heads x vdim rows gates every output value."""
+biases (on q, k, v and on the output projection), per-head temperature, the learned sink and the output gate are used when the
+checkpoint has them (none of them: plain causal softmax attention); a gate tensor of one row per head gates whole heads, one of
+heads x vdim rows gates every output value.  `out_tag` names the scratch buffer of the result, for a layer that runs two mixers side
+by side."""
 from __future__ import annotations
 
 import math
@@ -62,13 +64,15 @@ class WindowAttention:
 
     def __init__(self, model, key: str, layer_idx: int, *, heads: int, kv_heads: int, dim: int, vdim: int, window: int, pool: int,
                  rot_base: float, rot_dims: int, rot_scaling: dict | None, scale: float, rotate_values: bool = True,
-                 interleaved: bool = False, chunk: int = 0, softcap: float = 0.0, sink_one: bool = False, kv_from: int | None = None):
+                 interleaved: bool = False, chunk: int = 0, softcap: float = 0.0, sink_one: bool = False, kv_from: int | None = None,
+                 out_tag: str = "mix.y"):
         self.model, self.ext, self.key, self.layer_idx = model, model.ext, key, layer_idx
         self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
         self.window, self.pool, self.scale = window, pool, scale
         self.rot_base, self.rot_dims, self.rot_scaling = rot_base, rot_dims, rot_scaling
         self.rotate_values, self.interleaved = rotate_values, interleaved
         self.chunk, self.softcap, self.sink_one, self.kv_from = int(chunk), float(softcap), bool(sink_one), kv_from
+        self.out_tag = out_tag
         if heads % kv_heads or rot_dims > dim or rot_dims % 2 or (rotate_values and vdim % 2) or window <= 0 or pool < 0 \
                 or chunk < 0 or (chunk and pool) or softcap < 0:
             raise ValueError(f"{key}: inconsistent attention sizes")
@@ -80,7 +84,7 @@ class WindowAttention:
         H, G, dim, vd, width, f32 = self.heads, self.kv_heads, self.dim, self.vdim, self.model.width, torch.float32
         dev = self.model.device
         own_kv = self.kv_from is None
-        q, g = get("q"), get("g")
+        q, g = get("q"), get("g", optional=True)
         parts, names = [q], ["q"]
         if own_kv:
             k, v = get("k"), get("v")
@@ -88,17 +92,18 @@ class WindowAttention:
                 raise RuntimeError(f"{self.key}: tensor shapes do not match the mixer's sizes")
             parts += [k, v]
             names += ["k", "v"]
-        self.gate_head = tuple(g.shape) == (H, width) and vd != 1
-        if tuple(q.shape) != (H * dim, width) or tuple(g.shape) not in ((H * vd, width), (H, width)):
+        self.gated = g is not None
+        self.gate_head = self.gated and tuple(g.shape) == (H, width) and vd != 1
+        if tuple(q.shape) != (H * dim, width) or (self.gated and tuple(g.shape) not in ((H * vd, width), (H, width))):
             raise RuntimeError(f"{self.key}: tensor shapes do not match the mixer's sizes")
         # one linear for everything that reads the layer input: [q | k | v | g]; the gate's columns start at a multiple of 4
-        pad = (-sum(p.shape[0] for p in parts)) % 4
+        pad = (-sum(p.shape[0] for p in parts)) % 4 if self.gated else 0
         if pad:
             parts.append(torch.zeros((pad, width), dtype=q.dtype, device=dev))
         self.off_k = H * dim
         self.off_v = self.off_k + (G * dim if own_kv else 0)
         self.off_g = sum(p.shape[0] for p in parts)
-        self.front = DenseLinear(self.ext, self.key + ".front", torch.cat(parts + [g], 0))
+        self.front = DenseLinear(self.ext, self.key + ".front", torch.cat(parts + ([g] if self.gated else []), 0))
         biases = [get(n + ".b", optional=True) for n in names]
         self.front_bias = None
         if any(b is not None for b in biases):
@@ -116,6 +121,8 @@ class WindowAttention:
         else:
             self.sink = sink.to(f32).contiguous() if sink is not None else None
         self.o = DenseLinear(self.ext, self.key + ".o", get("o"))
+        ob = get("o.b", optional=True)
+        self.o_bias = ob.to(f32).contiguous() if ob is not None else None
         if self.q_scale.numel() != H or (self.sink is not None and self.sink.numel() != H) or tuple(self.o.weight.shape) != (width, H * vd):
             raise RuntimeError(f"{self.key}: tensor shapes do not match the mixer's sizes")
         self.freq, self.amp = rotary_tables(self.rot_base, self.rot_dims, self.rot_scaling, dev) if self.rot_dims else \
@@ -152,7 +159,7 @@ class WindowAttention:
                           self.rot_dims, self.vfreq, self.rotate_values, self.interleaved, batch.row_seq, batch.row_pos, batch.block_table,
                           page, self.pool if own else 0, rows, H, G, dim, vd)
         o = m.buf("attn.o", (rows, H * vd), m.dtype)
-        common = (q, st.k, st.v, st.k_pool, st.v_pool, self.sink, f, ncat, self.off_g, self.vfreq, self.rotate_values, self.interleaved,
+        common = (q, st.k, st.v, st.k_pool, st.v_pool, self.sink, f if self.gated else None, ncat, self.off_g, self.vfreq, self.rotate_values, self.interleaved,
                   batch.row_seq, batch.row_pos, batch.block_table, page, self.pool, o)
         var = dict(chunk=self.chunk, softcap=self.softcap, gate_head=self.gate_head)
         reach = self.chunk or self.window                     # the most tokens a position sees
@@ -175,4 +182,4 @@ class WindowAttention:
                                       **var)
         else:
             ext.window_attn(*common, rows, H, G, dim, vd, self.window, **var)
-        return self.o.forward(o, rows, out=m.buf("mix.y", (rows, m.width), f32))
+        return self.o.forward(o, rows, out=m.buf(self.out_tag, (rows, m.width), f32), bias=self.o_bias)

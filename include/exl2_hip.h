@@ -588,6 +588,44 @@ int exl2_wkv_scan_chunked(const float* r, const float* k, const float* v, const 
                           int total_chunks, const int* row_seq, const int* row_pos, float* zbuf, float* dbuf,
                           int heads, int n_key, int n_val, float eps, void* stream);
 
+/* ---- sandwich-normed residual steps, a hashed token-pair embedding, two more epilogue-free recurrences (csrc/rowops.hip, ssm.hip,
+   gated_scan.hip).  n_g(v) = v in `groups` equal runs, each divided by sqrt(mean(run^2) + eps). */
+
+/* x[r] <- x[r] + mult * n_g(ya y[r] + yb y2[r] + sum_k moe_y[r * top + k]) w_out  (y, y2, moe_y nullable; nothing is added when all
+   are), then out[r] = n_g(x[r]) w_in (out nullable).  row_idx: output row r reads stream row row_idx[r] (no addition then).  conv_w
+   [width, taps] (nullable; steps whose spans are single rows only): out[r] = hn + sum_j conv_w[:, j] hn_(p - taps + 1 + j) over the
+   sequence's last normed rows, kept in tail fp32 [slots, taps - 1, width] and rolled here; rows in front of position 0 are zeros.
+   Weights in the operand dtype; out in the operand dtype or fp32. */
+int exl2_sandwich_norm(float* x, const float* y, float ya, const float* y2, float yb, const float* moe_y, int top,
+                       const void* w_out, float mult, const void* w_in, void* out, int out_f32, const int* row_idx,
+                       const void* conv_w, float* tail, const int* row_seq, const int* row_pos, int taps, int dtype, int rows,
+                       int width, int groups, float eps, void* stream);
+/* x[r] = n_g(table[ids[r]] * scale + pair[(t' * mul_prev + ids[r] * mul_cur) mod buckets]) w, t' = the previous token of the row's
+   sequence (the row in front within a span, else prev_tok[slot]); row `buckets` of pair at position 0.  Afterwards prev_tok holds
+   every span's last token.  pair and w nullable (no pair term / no norm). */
+int exl2_embed_pair(const void* table, const void* pair, const void* w, const int* ids, int* prev_tok, const int* row_seq,
+                    const int* row_pos, const int* span_row0, const int* span_rows, int spans, int max_span_rows, float* x,
+                    int dtype, int rows, int width, int vocab, int buckets, int mul_prev, int mul_cur, float scale, int groups,
+                    float eps, void* stream);
+/* exl2_conv_silu_rows with a choice of output: residual 0: silu(conv + bias); 1: in + conv + bias without activation.  out fp32
+   (out_f32 = 1) or the operand dtype. */
+int exl2_conv_rows_ex(const float* in, int ld, const void* w, const void* bias, void* out, int ldo, int out_f32, int residual,
+                      float* tail, const int* span_row0, const int* span_rows, int spans, int max_span_rows,
+                      const int* row_seq, const int* row_pos, int dtype, int channels, int taps, void* stream);
+/* Linear attention over a matrix state S fp32 [slots, heads, n_key, n_val] per head and row.
+   mode 0: f = lower + (1 - lower) sigmoid(k), qq = silu(q); S <- diag(f) S + (1 - f) v^T; o = S^T qq.  q, k [rows, ld*] head h at
+           h * n_key; lower fp32 [heads * n_key]; qk_heads = heads.
+   mode 1: qq = q / sqrt(sum q^2 + 1e-6) * q_scale, kk = k / sqrt(sum k^2 + 1e-6) per head (q / k head h / (heads / qk_heads));
+           b = sigmoid(beta[h]); g = exp(-exp(a_log[h]) softplus(dt[h] + dt_bias[h])); S <- g S; u = b (v - S^T kk); S <- S + kk u^T;
+           o = S^T qq.
+   out = o / sqrt(mean(o^2) + eps) * norm_w (fp32 [n_val]) (* silu(gate), head h at h * n_val; nullable); [rows, ldo] operand dtype
+   (bfloat16) or fp32.  The state is read at a span's start (unless it starts at position 0) and written at its end. */
+int exl2_gated_scan(int mode, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* gate,
+                    int ldg, const float* beta, int ldb, const float* dt, int lddt, const float* dt_bias, const float* a_log,
+                    const float* lower, const float* norm_w, void* out, int ldo, int out_f32, float* state,
+                    const int* span_row0, const int* span_rows, int spans, const int* row_seq, const int* row_pos, int heads,
+                    int qk_heads, int n_key, int n_val, float q_scale, float eps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
