@@ -61,11 +61,12 @@ def parse():
     p.add_argument("--windows", type=int, default=5, help="timed windows of --steps steps (each after --warmup untimed steps from the same "
                                                            "cache position); the MEDIAN window is the reported value")
     p.add_argument("--headline-only", action="store_true", help="= --no-cpu-baseline --no-prefill --no-dropin --no-ctx-window (A/B runs)")
-    p.add_argument("--design", default=None, choices=["benolix", "tibalorn", "negilorn"],
+    p.add_argument("--design", default=None, choices=["benolix", "tibalorn", "negilorn", "kilurax"],
                    help="instead of the headline: prefill / decode throughput of a layer-stack design at real layer sizes beside the "
                         "package's closest other model of equal size (benolix: latent attention + MoE beside the quantized Mixtral-style "
                         "stack; tibalorn: state-space + windowed attention beside a latent-attention stack; negilorn: chunked attention + decaying "
-                        "linear attention + sigmoid MoE beside a state-space / windowed-attention stack; "
+                        "linear attention + sigmoid MoE beside a state-space / windowed-attention stack; kilurax: attention beside a state-space scan, "
+                        "forget-gate linear attention and gated delta rule behind sandwich norms beside a negilorn stack; "
                         "exllamav2_amd/bench_layered.py); one JSON line each")
     p.add_argument("--design-sizes", default="w2048,w4096")
     p.add_argument("--design-no-peer", action="store_true", help="--design: skip the peer model")

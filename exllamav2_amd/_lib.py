@@ -146,6 +146,9 @@ PROTOTYPES = {
     "exl2_conv_rows_ex": (ci, [vp, ci, vp, vp, vp, ci, ci, ci, vp, vp, vp, ci, ci, vp, vp, ci, ci, ci, vp]),
     "exl2_gated_scan": (ci, [ci, vp, ci, vp, ci, vp, ci, vp, ci, vp, ci, vp, ci, vp, vp, vp, vp, vp, ci, ci, vp, vp, vp, ci, vp, vp, ci, ci,
                              ci, ci, cf, cf, vp]),
+    "exl2_gated_scan_cols_supported": (ci, [ci, ci]),
+    "exl2_gated_scan_cols": (ci, [ci, vp, ci, vp, ci, vp, ci, vp, ci, vp, ci, vp, ci, vp, vp, vp, vp, vp, ci, ci, vp, vp, vp, ci, vp, vp, ci, vp,
+                                  ci, ci, ci, ci, cf, cf, vp]),
     # graphs
     "exl2_graph_begin_capture": (ci, [vp]),
     "exl2_graph_end_capture": (ci, [vp, C.POINTER(vp)]),

@@ -394,8 +394,127 @@ def bench_shift_peer(size: str, device="cuda:0", prompt: int = 2048, ctx: int = 
     return _bench_engine(model, out, s["vocab"], prompt, ctx, decode_steps, batches)
 
 
+SANDWICH_SIZES = {
+    # pattern: p = softmax attention beside a state-space scan, h = linear attention whose forget gate writes, d = gated delta rule;
+    # every layer has a sparse feed-forward with a shared expert
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=128, ssm_heads=32, ssm_vdim=64, state=128, la_heads=16, la_kv_heads=8,
+                  la_dim=128, la_vdim=128, experts=8, top=2, expert_ff=2816, shared_ff=2816, pattern="phdp", vocab=32000),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, ssm_heads=64, ssm_vdim=64, state=128, la_heads=32, la_kv_heads=16,
+                  la_dim=128, la_vdim=128, experts=8, top=2, expert_ff=7168, shared_ff=7168, pattern="phd", vocab=32000),
+}
+
+
+def sandwich_config(s: dict) -> dict:
+    layers = []
+    for ch in s["pattern"]:
+        ff = {"expert": {"ff": s["expert_ff"]}, "kind": "moe", "router": {"experts": s["experts"], "top": s["top"]}, "shared": {"ff": s["shared_ff"]}}
+        if ch == "p":
+            m = {"left": {"dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv_heads"], "vdim": s["vdim"], "scale": s["dim"] ** -0.5,
+                          "rot": {"base": 500000.0, "dims": s["dim"]}}, "left_scale": 1.0,
+                 "right": {"conv": 4, "groups": 1, "heads": s["ssm_heads"], "norm_groups": 1, "state": s["state"], "vdim": s["ssm_vdim"]},
+                 "right_scale": 1.0}
+            layers.append({"type": "parallel", "mixer": m, "mlp": ff})
+        elif ch == "h":
+            layers.append({"type": "hgrn2", "mixer": {"dim": s["la_dim"], "heads": s["la_heads"], "vdim": s["la_vdim"]}, "mlp": ff})
+        else:
+            layers.append({"type": "delta", "mixer": {"conv": 4, "dim": s["la_dim"], "heads": s["la_heads"], "kv_heads": s["la_kv_heads"],
+                                                      "vdim": s["la_vdim"]}, "mlp": ff})
+    return {"architecture": "Kilurax", "canon": {"taps": 4}, "embedding": {"bigram": {"buckets": 65521, "mul_cur": 7, "mul_prev": 127}, "scale": 1.0},
+            "layers": layers, "norm": {"eps": 1e-6, "groups": 2}, "residual_mult": 0.5, "vocab": s["vocab"], "width": s["width"]}
+
+
+def sandwich_random_tensors(cfg: dict, device, seed: int = 0) -> dict:
+    g = torch.Generator(device=device).manual_seed(seed)
+    T = {}
+
+    def mat(name, out, inp, gain=1.0):
+        T[name] = (torch.randn((out, inp), device=device, generator=g) * gain / inp ** 0.5).to(torch.bfloat16)
+
+    def vec(name, n, centre, spread=0.1):
+        T[name] = (centre + spread * torch.randn((n,), device=device, generator=g)).to(torch.bfloat16)
+
+    w, taps = cfg["width"], cfg["canon"]["taps"]
+    T["embed"] = (torch.randn((cfg["vocab"], w), device=device, generator=g) * 0.5).to(torch.bfloat16)
+    T["bigram"] = (torch.randn((cfg["embedding"]["bigram"]["buckets"] + 1, w), device=device, generator=g) * 0.5).to(torch.bfloat16)
+    vec("embed.norm", w, 1.0); vec("final.norm", w, 1.0); mat("head", cfg["vocab"], w)
+    for i, L in enumerate(cfg["layers"]):
+        m, k = L["mixer"], f"l{i}"
+        for n in ("norm1", "norm1b", "norm2", "norm2b"):
+            vec(f"{k}.{n}", w, 1.0)
+        for n in ("canon1", "canon2"):
+            T[f"{k}.{n}"] = (0.2 * torch.randn((w, taps), device=device, generator=g)).to(torch.bfloat16)
+        if L["type"] == "parallel":
+            a, r = m["left"], m["right"]
+            H, G, dim, vd = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            mat(k + ".mix.left.q", H * dim, w); mat(k + ".mix.left.k", G * dim, w); mat(k + ".mix.left.v", G * vd, w); mat(k + ".mix.left.o", w, H * vd)
+            vec(k + ".mix.left.q.b", H * dim, 0.0); vec(k + ".mix.left.k.b", G * dim, 0.0); vec(k + ".mix.left.v.b", G * vd, 0.0); vec(k + ".mix.left.o.b", w, 0.0)
+            inner, gn = r["heads"] * r["vdim"], r["groups"] * r["state"]
+            mat(k + ".mix.right.in", 2 * inner + 2 * gn + r["heads"], w)
+            T[k + ".mix.right.conv"] = (0.5 * torch.randn((inner + 2 * gn, r["conv"]), device=device, generator=g)).to(torch.bfloat16)
+            vec(k + ".mix.right.conv.b", inner + 2 * gn, 0.0); vec(k + ".mix.right.dt_bias", r["heads"], -1.0, 0.5)
+            vec(k + ".mix.right.A_log", r["heads"], 0.0, 0.5); vec(k + ".mix.right.D", r["heads"], 1.0)
+            vec(k + ".mix.right.norm", inner, 1.0); mat(k + ".mix.right.o", w, inner)
+        elif L["type"] == "hgrn2":
+            H, dim, vd = m["heads"], m["dim"], m["vdim"]
+            mat(k + ".mix.q", H * dim, w); mat(k + ".mix.f", H * dim, w); mat(k + ".mix.v", H * vd, w); vec(k + ".mix.f.b", H * dim, 1.0, 1.0)
+            T[k + ".mix.lower"] = (0.9 * torch.rand((H * dim,), device=device, generator=g)).to(torch.bfloat16)
+            vec(k + ".mix.norm", vd, 1.0); mat(k + ".mix.o", w, H * vd)
+        else:
+            H, G, dim, vd = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            mat(k + ".mix.q", G * dim, w); mat(k + ".mix.k", G * dim, w); mat(k + ".mix.v", H * vd, w)
+            for n, c in (("q", G * dim), ("k", G * dim), ("v", H * vd)):
+                T[f"{k}.mix.{n}.conv"] = (0.5 * torch.randn((c, m["conv"]), device=device, generator=g)).to(torch.bfloat16)
+            mat(k + ".mix.b", H, w); mat(k + ".mix.a", H, w); mat(k + ".mix.g", H * vd, w)
+            vec(k + ".mix.dt_bias", H, -1.0, 0.5); vec(k + ".mix.A_log", H, -1.0, 0.5); vec(k + ".mix.norm", vd, 1.0); mat(k + ".mix.o", w, H * vd)
+        ms = L["mlp"]
+        mat(k + ".mlp.router", ms["router"]["experts"], w)
+        for n, ff in [(f"e{e}", ms["expert"]["ff"]) for e in range(ms["router"]["experts"])] + [("shared", ms["shared"]["ff"])]:
+            mat(f"{k}.mlp.{n}.gate", ff, w); mat(f"{k}.mlp.{n}.up", ff, w); mat(f"{k}.mlp.{n}.down", w, ff)
+    return T
+
+
+def bench_sandwich(size: str, device="cuda:0", prompt: int = 2048, ctx: int = 1024, decode_steps: int = 64, batches=(1, 4)) -> dict:
+    from .config import LayeredConfig
+    from .layered import LayeredModel
+    s = SANDWICH_SIZES[size]
+    cfg = sandwich_config(s)
+    model = LayeredModel(LayeredConfig.from_dict_sandwich(cfg), device=device, dtype=torch.bfloat16).load(sandwich_random_tensors(cfg, device))
+    out = {"design": "kilurax", "size": size, "layers": len(cfg["layers"]), "pattern": s["pattern"], "weight_bytes_per_token": model.weight_bytes()}
+    return _bench_engine(model, out, s["vocab"], prompt, ctx, decode_steps, batches)
+
+
+def bench_sandwich_peer(size: str, device="cuda:0", prompt: int = 2048, ctx: int = 1024, decode_steps: int = 64, batches=(1, 4)) -> dict:
+    """the closest model of the package: a token-shifted stack of chunked attention and decaying linear attention (bfloat16, the same
+    engine) of the same width and depth -- an attention layer of the same heads (one chunk over the whole context) for every layer of
+    attention beside a state-space scan, a decaying linear attention of the same state size per head for every other linear-attention
+    layer, the same sparse feed-forward (two-matrix experts half as wide again, so that a token streams the same bytes)"""
+    from .config import LayeredConfig
+    from .layered import LayeredModel
+    s = SANDWICH_SIZES[size]
+    layers = []
+    for ch in s["pattern"]:
+        ff = {"expert": {"ff": s["expert_ff"] * 3 // 2}, "kind": "moe", "router": {"experts": s["experts"], "top": s["top"]},
+              "shared": {"ff": s["shared_ff"] * 3 // 2}}
+        if ch == "p":
+            m = {"dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv_heads"], "vdim": s["vdim"], "mask": {"size": 1 << 20},
+                 "scale": s["dim"] ** -0.5, "softcap": 30.0, "rot": {"base": 500000.0, "dims": s["dim"]}}
+            layers.append({"type": "attention", "mlp": ff, "mixer": m})
+        else:
+            layers.append({"type": "wkv", "mlp": ff, "mixer": {"dim": s["la_dim"], "heads": s["la_heads"]}})
+    cfg = {"architecture": "Negilorn", "layers": layers, "logit_scale": 0.5, "norm": {"eps": 1e-5}, "vocab": s["vocab"], "width": s["width"]}
+    model = LayeredModel(LayeredConfig.from_dict_prerms_shift(cfg), device=device, dtype=torch.bfloat16).load(
+        shift_random_tensors(cfg, dict(rank=64), device))
+    out = {"design": "negilorn-peer", "size": size, "layers": len(layers), "weight_bytes_per_token": model.weight_bytes()}
+    return _bench_engine(model, out, s["vocab"], prompt, ctx, decode_steps, batches)
+
+
 def run(sizes, device="cuda:0", peer: bool = True, design: str = "benolix"):
     for size in sizes:
+        if design == "kilurax":
+            print(json.dumps(bench_sandwich(size, device)), flush=True)
+            if peer:
+                print(json.dumps(bench_sandwich_peer(size, device)), flush=True)
+            continue
         if design == "negilorn":
             print(json.dumps(bench_shift(size, device)), flush=True)
             if peer:

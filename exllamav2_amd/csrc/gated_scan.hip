@@ -192,6 +192,205 @@ KERNEL void __launch_bounds__(256) gated_scan_kernel(const GatedScanArgs a)
     }
 }
 
+// ---- the same recurrences for portions of prompts: columns of the state dealt to workgroups -------------------------------------------
+// The value columns of a head's state never meet inside the recurrence (u_p = beta (v_p - S[:, p] . k), o_p = S[:, p] . q), so a
+// span's walk is dealt to (head, block of GSC_COLS columns) workgroups: GSC_KS = 16 lanes share a column, each holds N / 16 rows in
+// registers, and a token costs a thread a handful of fused multiply-adds and four lane exchanges per sum instead of a pass over
+// N / 2 rows.  Tokens are taken GSC_CHUNK at a time; the raw projections of the NEXT round are requested into registers before a round
+// is stepped through, so their latency hides behind it, and turned into gates / unit vectors / decays when they are written to LDS.
+// The raw read-out goes to o_raw fp32 [rows, heads * P]; the head norm needs the whole head and is head_norm_gate_kernel's.
+
+#define GSC_KS 16
+#define GSC_COLS 16                          // 256 threads = 16 columns x 16 lanes
+#define GSC_CHUNK 32
+#define GSC_TPW (GSC_CHUNK / 4)              // tokens a wave stages per round
+#define GSC_MAX_N 256                        // key channels: 4 per lane while a wave stages a token, NPT = N / 16 <= 16 rows per thread
+
+template <int NPT, int MODE>
+KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a, float* o_raw)
+{
+    DYN_SMEM(smem);
+    const int h = bid_x(), sp = bid_y(), cb = bid_z();
+    const int n_tok = a.span_rows[sp], r0 = a.span_row0[sp];
+    const int pos0 = a.row_pos[r0];
+    const int P = a.P, N = a.N;
+    const int t = tid(), lane = lane_id(), wv = wave_id();
+    const int pl = t / GSC_KS, j = t % GSC_KS;
+    const int p = cb * GSC_COLS + pl;
+    const bool owner = p < P;
+    const int pc = owner ? p : P - 1;
+    const int hq = h / (a.heads / a.qk_heads);
+    float* s_q = (float*)smem;                                   // [CHUNK, N]
+    float* s_k = s_q + GSC_CHUNK * N;                            // [CHUNK, N]
+    float* s_v = s_k + GSC_CHUNK * N;                            // [CHUNK, COLS]
+    float* s_b = s_v + GSC_CHUNK * GSC_COLS;                     // [CHUNK]
+    float* s_g = s_b + GSC_CHUNK;                                // [CHUNK]
+    float* st = a.state + ((long long)a.row_seq[r0] * a.heads + h) * (long long)N * P;
+    float S[NPT];
+    #pragma unroll
+    for (int i = 0; i < NPT; i++)
+    {
+        const int n = j + GSC_KS * i;
+        S[i] = (owner && pos0 > 0 && n < N) ? st[(long long)n * P + p] : 0.0f;
+    }
+    const float a_neg = MODE == GS_DELTA ? -expf(a.a_log[h]) : 0.0f, dtb = MODE == GS_DELTA ? a.dt_bias[h] : 0.0f;
+    // what a thread keeps of the next round while the current one is stepped through
+    float rq[GSC_TPW][GSC_MAX_N / 64], rk[GSC_TPW][GSC_MAX_N / 64], rv[2], rb = 0.0f, rd = 0.0f;
+    const int qh = MODE == GS_DELTA ? hq : h;
+
+    auto request = [&](int c0)
+    {
+        const int nc = min(GSC_CHUNK, n_tok - c0);
+        #pragma unroll
+        for (int u = 0; u < GSC_TPW; u++)
+        {
+            const int kk = wv + 4 * u;
+            const long long row = r0 + c0 + min(kk, nc - 1);
+            #pragma unroll
+            for (int e = 0; e < GSC_MAX_N / 64; e++)
+            {
+                const int n = lane + 64 * e;
+                rq[u][e] = n < N ? a.q[row * a.ldq + qh * N + n] : 0.0f;
+                rk[u][e] = n < N ? a.k[row * a.ldk + qh * N + n] : 0.0f;
+            }
+        }
+        #pragma unroll
+        for (int u = 0; u < 2; u++)
+        {
+            const int kk = t / GSC_COLS + 16 * u, col = cb * GSC_COLS + t % GSC_COLS;
+            rv[u] = (kk < nc && col < P) ? a.v[(long long)(r0 + c0 + kk) * a.ldv + h * P + col] : 0.0f;
+        }
+        if (MODE == GS_DELTA && t < GSC_CHUNK)
+        {
+            const long long row = r0 + c0 + min(t, nc - 1);
+            rb = a.beta[row * a.ldb + h];
+            rd = a.dt[row * a.lddt + h];
+        }
+    };
+
+    auto publish = [&]()
+    {
+        #pragma unroll
+        for (int u = 0; u < GSC_TPW; u++)
+        {
+            const int kk = wv + 4 * u;
+            if (MODE == GS_DELTA)
+            {
+                float sq = 0.0f, sk = 0.0f;
+                #pragma unroll
+                for (int e = 0; e < GSC_MAX_N / 64; e++) { sq = fmaf(rq[u][e], rq[u][e], sq); sk = fmaf(rk[u][e], rk[u][e], sk); }
+                sq = wave_allreduce_add(sq);
+                sk = wave_allreduce_add(sk);
+                const float mq = a.q_scale / sqrtf(sq + 1e-6f), mk = 1.0f / sqrtf(sk + 1e-6f);
+                #pragma unroll
+                for (int e = 0; e < GSC_MAX_N / 64; e++)
+                {
+                    const int n = lane + 64 * e;
+                    if (n < N) { s_q[kk * N + n] = rq[u][e] * mq; s_k[kk * N + n] = rk[u][e] * mk; }
+                }
+            }
+            else
+            {
+                #pragma unroll
+                for (int e = 0; e < GSC_MAX_N / 64; e++)
+                {
+                    const int n = lane + 64 * e;
+                    if (n < N)
+                    {
+                        const float lo = a.lower[h * N + n];
+                        s_q[kk * N + n] = rq[u][e] * gs_sigmoid(rq[u][e]);
+                        s_k[kk * N + n] = fmaf(1.0f - lo, gs_sigmoid(rk[u][e]), lo);
+                    }
+                }
+            }
+        }
+        #pragma unroll
+        for (int u = 0; u < 2; u++) s_v[(t / GSC_COLS + 16 * u) * GSC_COLS + t % GSC_COLS] = rv[u];
+        if (MODE == GS_DELTA && t < GSC_CHUNK)
+        {
+            s_b[t] = gs_sigmoid(rb);
+            s_g[t] = expf(a_neg * gs_softplus(rd + dtb));
+        }
+    };
+
+    request(0);
+    for (int c0 = 0; c0 < n_tok; c0 += GSC_CHUNK)
+    {
+        const int nc = min(GSC_CHUNK, n_tok - c0);
+        block_sync_lds();                                        // the round before has been stepped through by every thread
+        publish();
+        block_sync_lds();
+        if (c0 + GSC_CHUNK < n_tok) request(c0 + GSC_CHUNK);
+        for (int kk = 0; kk < nc; kk++)
+        {
+            const float vv = s_v[kk * GSC_COLS + pl];
+            float o = 0.0f;
+            if (MODE == GS_DELTA)
+            {
+                const float g = s_g[kk];
+                float kt = 0.0f;
+                #pragma unroll
+                for (int i = 0; i < NPT; i++)
+                {
+                    const int n = j + GSC_KS * i;
+                    if (n < N) { S[i] *= g; kt = fmaf(S[i], s_k[kk * N + n], kt); }
+                }
+                kt = row16_allreduce_add(kt);
+                const float u = s_b[kk] * (vv - kt);
+                #pragma unroll
+                for (int i = 0; i < NPT; i++)
+                {
+                    const int n = j + GSC_KS * i;
+                    if (n < N) { S[i] = fmaf(s_k[kk * N + n], u, S[i]); o = fmaf(S[i], s_q[kk * N + n], o); }
+                }
+            }
+            else
+            {
+                #pragma unroll
+                for (int i = 0; i < NPT; i++)
+                {
+                    const int n = j + GSC_KS * i;
+                    if (n < N)
+                    {
+                        const float f = s_k[kk * N + n];
+                        S[i] = fmaf(f, S[i], (1.0f - f) * vv);
+                        o = fmaf(S[i], s_q[kk * N + n], o);
+                    }
+                }
+            }
+            o = row16_allreduce_add(o);
+            if (owner && j == 0) o_raw[(long long)(r0 + c0 + kk) * a.heads * P + h * P + p] = o;
+        }
+    }
+    #pragma unroll
+    for (int i = 0; i < NPT; i++)
+    {
+        const int n = j + GSC_KS * i;
+        if (owner && n < N) st[(long long)n * P + p] = S[i];
+    }
+    (void)pc;
+}
+
+// grid (rows, heads), one wave: out = o / sqrt(mean(o^2) + eps) * norm_w (* silu(gate))
+template <typename T>
+KERNEL void __launch_bounds__(64) head_norm_gate_kernel(const float* o_raw, const float* norm_w, const float* gate, int ldg, void* out, int ldo,
+                                                         int heads, int P, float eps)
+{
+    const long long row = bid_x();
+    const int h = bid_y();
+    const float* o = o_raw + row * heads * P + h * P;
+    float ss = 0.0f;
+    for (int pp = lane_id(); pp < P; pp += 64) ss = fmaf(o[pp], o[pp], ss);
+    ss = wave_allreduce_add(ss);
+    const float rinv = 1.0f / sqrtf(ss / (float)P + eps);
+    for (int pp = lane_id(); pp < P; pp += 64)
+    {
+        float v = o[pp] * rinv * norm_w[pp];
+        if (gate) { const float gv = gate[row * ldg + h * P + pp]; v *= gv * gs_sigmoid(gv); }
+        gs_st<T>((T*)out + row * ldo + h * P + pp, v);
+    }
+}
+
 template <typename T, int MODE>
 static void gated_scan_launch(const GatedScanArgs& a, int npt, dim3 grid, dim3 block, size_t smem, void* stream)
 {
@@ -252,6 +451,65 @@ extern "C" int exl2_gated_scan(int mode, const float* q, int ldq, const float* k
         if (out_f32) gated_scan_launch<float, GS_FORGET_WRITES>(a, npt, grid, block, smem, stream);
         else gated_scan_launch<u16, GS_FORGET_WRITES>(a, npt, grid, block, smem, stream);
     }
+    HIP_TRY(hipGetLastError());
+    return EXL2_OK;
+}
+
+/* 1 if exl2_gated_scan_cols takes this state shape */
+extern "C" int exl2_gated_scan_cols_supported(int n_key, int n_val)
+{
+    return n_key > 0 && n_key <= GSC_MAX_N && n_val > 0 ? 1 : 0;
+}
+
+/* exl2_gated_scan for portions of prompts: a span's walk dealt to (head, 16 value columns) workgroups, the next round's inputs in
+   flight behind the current one; the head norm (and gate) as a second launch over o_raw (scratch, fp32 [rows, heads * n_val]).  Same
+   operands and results as exl2_gated_scan (sums associate differently: results agree to rounding). */
+extern "C" int exl2_gated_scan_cols(int mode, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* gate,
+                                    int ldg, const float* beta, int ldb, const float* dt, int lddt, const float* dt_bias,
+                                    const float* a_log, const float* lower, const float* norm_w, void* out, int ldo, int out_f32,
+                                    float* state, const int* span_row0, const int* span_rows, int spans, const int* row_seq,
+                                    const int* row_pos, int rows, float* o_raw, int heads, int qk_heads, int n_key, int n_val,
+                                    float q_scale, float eps, void* stream)
+{
+    EXL2_REQUIRE(mode == GS_FORGET_WRITES || mode == GS_DELTA, "gated_scan_cols: mode must be 0 (forget gate writes) or 1 (delta rule)");
+    EXL2_REQUIRE(q && k && v && norm_w && out && state && o_raw && span_row0 && span_rows && row_seq && row_pos, "gated_scan_cols: null operand");
+    EXL2_REQUIRE(mode != GS_FORGET_WRITES || lower, "gated_scan_cols: the forget gate needs its lower bound");
+    EXL2_REQUIRE(mode != GS_DELTA || (beta && dt && dt_bias && a_log), "gated_scan_cols: the delta rule needs beta and the decay's inputs");
+    EXL2_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && (mode == GS_DELTA || qk_heads == heads), "gated_scan_cols: %d heads over %d query / key heads", heads, qk_heads);
+    EXL2_REQUIRE(exl2_gated_scan_cols_supported(n_key, n_val), "gated_scan_cols: state %d x %d", n_key, n_val);
+    if (spans <= 0 || rows <= 0) return EXL2_OK;
+    GatedScanArgs a;
+    a.q = q; a.ldq = ldq; a.k = k; a.ldk = ldk; a.v = v; a.ldv = ldv; a.gate = gate; a.ldg = ldg; a.beta = beta; a.ldb = ldb; a.dt = dt;
+    a.lddt = lddt; a.dt_bias = dt_bias; a.a_log = a_log; a.lower = lower; a.norm_w = norm_w; a.out = out; a.ldo = ldo; a.state = state;
+    a.span_row0 = span_row0; a.span_rows = span_rows; a.row_seq = row_seq; a.row_pos = row_pos;
+    a.heads = heads; a.qk_heads = qk_heads; a.N = n_key; a.P = n_val; a.KS = GSC_KS; a.q_scale = q_scale; a.eps = eps;
+    const size_t smem = sizeof(float) * ((size_t)GSC_CHUNK * (2 * n_key + GSC_COLS + 2));
+    if (smem > 48 * 1024)
+    {
+        static bool attr_done[EXL2_MAX_DEVICES];
+        if (exl2_first_on_device(attr_done))
+        {
+            (void)hipFuncSetAttribute((const void*)gated_scan_cols_kernel<16, GS_FORGET_WRITES>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_cols_kernel<16, GS_DELTA>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        }
+    }
+    const dim3 grid(heads, spans, (n_val + GSC_COLS - 1) / GSC_COLS);
+    const int npt = (n_key + GSC_KS - 1) / GSC_KS;
+    if (mode == GS_DELTA)
+    {
+        if (npt <= 4) LAUNCH((gated_scan_cols_kernel<4, GS_DELTA>), grid, dim3(256), smem, stream, a, o_raw);
+        else if (npt <= 8) LAUNCH((gated_scan_cols_kernel<8, GS_DELTA>), grid, dim3(256), smem, stream, a, o_raw);
+        else LAUNCH((gated_scan_cols_kernel<16, GS_DELTA>), grid, dim3(256), smem, stream, a, o_raw);
+    }
+    else
+    {
+        if (npt <= 4) LAUNCH((gated_scan_cols_kernel<4, GS_FORGET_WRITES>), grid, dim3(256), smem, stream, a, o_raw);
+        else if (npt <= 8) LAUNCH((gated_scan_cols_kernel<8, GS_FORGET_WRITES>), grid, dim3(256), smem, stream, a, o_raw);
+        else LAUNCH((gated_scan_cols_kernel<16, GS_FORGET_WRITES>), grid, dim3(256), smem, stream, a, o_raw);
+    }
+    const float* gt = mode == GS_DELTA ? gate : nullptr;
+    if (out_f32) LAUNCH(head_norm_gate_kernel<float>, dim3(rows, heads), dim3(64), 0, stream, (const float*)o_raw, norm_w, gt, ldg, out, ldo, heads, n_val, eps);
+    else LAUNCH(head_norm_gate_kernel<u16>, dim3(rows, heads), dim3(64), 0, stream, (const float*)o_raw, norm_w, gt, ldg, out, ldo, heads, n_val, eps);
     HIP_TRY(hipGetLastError());
     return EXL2_OK;
 }

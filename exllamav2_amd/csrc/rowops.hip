@@ -410,6 +410,140 @@ KERNEL void __launch_bounds__(256) sandwich_norm_kernel(const SandwichArgs a)
     }
 }
 
+// The same step for rows of up to 256 * 4 * NC values in fours, up to SW_MAX_GROUPS norm groups of a multiple of four values and
+// up to SW_MAX_TAPS taps: a thread keeps its values in registers, every operand of the launch -- the sublayer's outputs, the stream,
+// both weights, the convolution's weights and the slot's tail -- is requested before the first is used, and the sums of all groups
+// close in ONE exchange through LDS per norm.
+#define SW_MAX_GROUPS 8
+#define SW_MAX_TAPS 4
+
+template <int NC>
+DEV void sw_group_sums(const f32x4* v, const int* grp, const bool* live, int groups, float* part, float* sums)
+{
+    float ss[SW_MAX_GROUPS];
+    #pragma unroll
+    for (int g = 0; g < SW_MAX_GROUPS; g++) ss[g] = 0.0f;
+    #pragma unroll
+    for (int e = 0; e < NC; e++)
+    {
+        const float q = live[e] ? (v[e][0] * v[e][0] + v[e][1] * v[e][1]) + (v[e][2] * v[e][2] + v[e][3] * v[e][3]) : 0.0f;
+        #pragma unroll
+        for (int g = 0; g < SW_MAX_GROUPS; g++) ss[g] += grp[e] == g ? q : 0.0f;
+    }
+    block_sync();                                                // the exchange buffer may still be read from the norm before
+    #pragma unroll
+    for (int g = 0; g < SW_MAX_GROUPS; g++)
+        if (g < groups)
+        {
+            const float w = wave_allreduce_add(ss[g]);
+            if (lane_id() == 0) part[wave_id() * SW_MAX_GROUPS + g] = w;
+        }
+    block_sync();
+    #pragma unroll
+    for (int g = 0; g < SW_MAX_GROUPS; g++)
+        sums[g] = g < groups ? (part[g] + part[SW_MAX_GROUPS + g]) + (part[2 * SW_MAX_GROUPS + g] + part[3 * SW_MAX_GROUPS + g]) : 0.0f;
+}
+
+template <typename T, int NC>
+KERNEL void __launch_bounds__(256) sandwich_norm_vec_kernel(const SandwichArgs a)
+{
+    SHARED float part[4 * SW_MAX_GROUPS];
+    const int r = bid_x();
+    const long long src = a.row_idx ? a.row_idx[r] : r;
+    float* xr = a.x + src * a.width;
+    const int gs = a.width / a.groups;
+    const bool pending = a.y || a.y2 || a.moe_y;
+    const bool conv = a.conv_w != nullptr;
+    f32x4 xv[NC], tv[NC], wo[NC], wi[NC], tl[NC][SW_MAX_TAPS - 1];
+    float cw[NC][4][SW_MAX_TAPS];
+    int grp[NC]; bool live[NC];
+    float* tail = nullptr; int pos = 0;
+    if (conv && a.taps > 1) { tail = a.tail + (long long)a.row_seq[r] * (a.taps - 1) * a.width; pos = a.row_pos[r]; }
+    const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    #pragma unroll
+    for (int e = 0; e < NC; e++)
+    {
+        const int i = 4 * (tid() + 256 * e);
+        live[e] = i < a.width;
+        grp[e] = live[e] ? i / gs : -1;
+        xv[e] = tv[e] = wo[e] = wi[e] = zero4;
+        if (!live[e]) continue;
+        xv[e] = *(const f32x4*)(xr + i);
+        if (pending)
+        {
+            wo[e] = ro_ld4<T>((const T*)a.w_out + i);
+            if (a.y) { const f32x4 y = *(const f32x4*)(a.y + src * a.width + i); tv[e] = a.ya * y; }
+            if (a.y2) { const f32x4 y = *(const f32x4*)(a.y2 + src * a.width + i); tv[e] += a.yb * y; }
+            for (int k = 0; k < (a.moe_y ? a.top : 0); k++) tv[e] += *(const f32x4*)(a.moe_y + (src * a.top + k) * a.width + i);
+        }
+        if (a.out) wi[e] = ro_ld4<T>((const T*)a.w_in + i);
+        if (conv)
+        {
+            #pragma unroll
+            for (int k = 0; k < 4; k++)
+                #pragma unroll
+                for (int j = 0; j < SW_MAX_TAPS; j++)
+                    cw[e][k][j] = j < a.taps ? ro_ld<T>((const T*)a.conv_w + (long long)(i + k) * a.taps + j) : 0.0f;
+            #pragma unroll
+            for (int j = 0; j < SW_MAX_TAPS - 1; j++)
+                tl[e][j] = (j < a.taps - 1 && pos - (a.taps - 1 - j) >= 0) ? *(const f32x4*)(tail + (long long)j * a.width + i) : zero4;
+        }
+    }
+    float sums[SW_MAX_GROUPS];
+    if (pending)
+    {
+        sw_group_sums<NC>(tv, grp, live, a.groups, part, sums);
+        #pragma unroll
+        for (int e = 0; e < NC; e++)
+        {
+            if (!live[e]) continue;
+            float s = 0.0f;
+            #pragma unroll
+            for (int g = 0; g < SW_MAX_GROUPS; g++) s = grp[e] == g ? sums[g] : s;
+            const float mul = a.mult / sqrtf(s / (float)gs + a.eps);
+            #pragma unroll
+            for (int k = 0; k < 4; k++) xv[e][k] = fmaf(tv[e][k] * mul, wo[e][k], xv[e][k]);
+            *(f32x4*)(xr + 4 * (tid() + 256 * e)) = xv[e];
+        }
+    }
+    if (!a.out) return;
+    sw_group_sums<NC>(xv, grp, live, a.groups, part, sums);
+    #pragma unroll
+    for (int e = 0; e < NC; e++)
+    {
+        if (!live[e]) continue;
+        const int i = 4 * (tid() + 256 * e);
+        float s = 0.0f;
+        #pragma unroll
+        for (int g = 0; g < SW_MAX_GROUPS; g++) s = grp[e] == g ? sums[g] : s;
+        const float rinv = 1.0f / sqrtf(s / (float)gs + a.eps);
+        f32x4 hn, o;
+        #pragma unroll
+        for (int k = 0; k < 4; k++) hn[k] = xv[e][k] * rinv * wi[e][k];
+        o = hn;
+        if (conv)
+        {
+            #pragma unroll
+            for (int k = 0; k < 4; k++)
+            {
+                float acc = 0.0f;
+                #pragma unroll
+                for (int j = 0; j < SW_MAX_TAPS; j++)
+                    if (j < a.taps) acc = fmaf(cw[e][k][j], j == a.taps - 1 ? hn[k] : tl[e][j < SW_MAX_TAPS - 1 ? j : 0][k], acc);
+                o[k] = hn[k] + acc;
+            }
+            // the tail moves up by one row: entry j takes entry j + 1, the newest takes this row
+            #pragma unroll
+            for (int j = 0; j < SW_MAX_TAPS - 1; j++)
+                if (j < a.taps - 1)
+                    *(f32x4*)(tail + (long long)j * a.width + i) = j == a.taps - 2 ? hn : tl[e][j + 1 < SW_MAX_TAPS - 1 ? j + 1 : 0];
+        }
+        if (a.out_f32) *(f32x4*)((float*)a.out + (long long)r * a.width + i) = o;
+        else *(u32x2*)((u16*)a.out + (long long)r * a.width + i) =
+                 (u32x2){(u32)f32_to_bf16(o[0]) | ((u32)f32_to_bf16(o[1]) << 16), (u32)f32_to_bf16(o[2]) | ((u32)f32_to_bf16(o[3]) << 16)};
+    }
+}
+
 // ---- token embedding + hashed token-pair embedding + norm ------------------------------------------------------------------------
 // x = n_g(table[t] * scale + pair[(t' mul_prev + t mul_cur) mod buckets]) w, t' = the sequence's previous token: the row in front
 // when that belongs to the same sequence, else what the slot keeps (prev_tok int32 [slots]); row `buckets` of the pair table at
@@ -788,6 +922,27 @@ extern "C" int exl2_sandwich_norm(float* x, const float* y, float ya, const floa
     a.x = x; a.y = y; a.ya = ya; a.y2 = y2; a.yb = yb; a.moe_y = moe_y; a.top = top; a.w_out = w_out; a.mult = mult; a.w_in = w_in;
     a.out = out; a.out_f32 = out_f32 || dtype == 1; a.row_idx = row_idx; a.conv_w = conv_w; a.tail = tail; a.row_seq = row_seq;
     a.row_pos = row_pos; a.taps = taps; a.width = width; a.groups = groups; a.eps = eps;
+    const auto al16 = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
+    const bool vec = width % 4 == 0 && width <= 256 * 4 * 4 && (width / groups) % 4 == 0 && groups <= SW_MAX_GROUPS && taps <= SW_MAX_TAPS
+                     && al16(x) && al16(y) && al16(y2) && al16(moe_y) && al16(w_out) && al16(w_in) && al16(out) && al16(tail) && (dtype == 0 || al16(w_in));
+    if (vec)
+    {
+        const int nc = width <= 1024 ? 1 : width <= 2048 ? 2 : 4;
+        if (dtype == 0)
+        {
+            if (nc == 1) LAUNCH((sandwich_norm_vec_kernel<u16, 1>), dim3(rows), dim3(256), 0, stream, a);
+            else if (nc == 2) LAUNCH((sandwich_norm_vec_kernel<u16, 2>), dim3(rows), dim3(256), 0, stream, a);
+            else LAUNCH((sandwich_norm_vec_kernel<u16, 4>), dim3(rows), dim3(256), 0, stream, a);
+        }
+        else
+        {
+            if (nc == 1) LAUNCH((sandwich_norm_vec_kernel<float, 1>), dim3(rows), dim3(256), 0, stream, a);
+            else if (nc == 2) LAUNCH((sandwich_norm_vec_kernel<float, 2>), dim3(rows), dim3(256), 0, stream, a);
+            else LAUNCH((sandwich_norm_vec_kernel<float, 4>), dim3(rows), dim3(256), 0, stream, a);
+        }
+        HIP_TRY(hipGetLastError());
+        return EXL2_OK;
+    }
     const size_t smem = (size_t)width * 4;
     if (smem > 48 * 1024)
     {

@@ -1117,8 +1117,9 @@ class ExtC:
 
     def gated_scan(self, mode: int, f, ld: int, q_off: int, k_off: int, v, ldv: int, v_off: int, norm_w, out, state, spans, row_seq, row_pos,
                    heads: int, qk_heads: int, n_key: int, n_val: int, eps: float, q_scale: float = 1.0, lower=None, gate_off: int | None = None,
-                   beta_off: int = 0, dt_off: int = 0, dt_bias=None, a_log=None, qk=None, ldqk: int = 0) -> None:
-        """f fp32 [rows, ld]: the mixer's projections -- mode 0: q pre-activation at q_off, forget-gate pre-activation at k_off; mode 1:
+                   beta_off: int = 0, dt_off: int = 0, dt_bias=None, a_log=None, qk=None, ldqk: int = 0, o_raw=None) -> None:
+        """o_raw (fp32 scratch [rows, heads * n_val]) given: the form for portions of prompts (exl2_gated_scan_cols).
+        f fp32 [rows, ld]: the mixer's projections -- mode 0: q pre-activation at q_off, forget-gate pre-activation at k_off; mode 1:
         beta / decay inputs / output gate at beta_off / dt_off / gate_off, q and k in `qk` fp32 [rows, ldqk] at q_off / k_off (the
         convolved rows).  v fp32 [rows, ldv] at v_off.  out [rows, heads * n_val] operand dtype or fp32."""
         row0, nrows, n, _longest = spans
@@ -1126,15 +1127,24 @@ class ExtC:
         pqk = self._ptr(qk, torch.float32, "qk") if qk is not None else pf
         lqk = int(ldqk) if qk is not None else int(ld)
         delta = mode == self.SCAN_DELTA
-        self.lib.check(self.lib.exl2_gated_scan(
-            int(mode), pqk + q_off * 4, lqk, pqk + k_off * 4, lqk, self._ptr(v, torch.float32, "v") + v_off * 4, int(ldv),
-            (pf + gate_off * 4) if gate_off is not None else None, int(ld), (pf + beta_off * 4) if delta else None, int(ld),
-            (pf + dt_off * 4) if delta else None, int(ld), self._ptr(dt_bias, torch.float32, "dt_bias"),
-            self._ptr(a_log, torch.float32, "a_log"), self._ptr(lower, torch.float32, "lower"), self._ptr(norm_w, torch.float32, "norm_w"),
-            self._ptr(out, None, "out"), out.shape[-1], int(out.dtype is torch.float32), self._ptr(state, torch.float32, "state"),
-            self._ptr(row0, torch.int32, "span_row0"), self._ptr(nrows, torch.int32, "span_rows"), int(n),
-            self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"), int(heads), int(qk_heads), int(n_key),
-            int(n_val), float(q_scale), float(eps), self._stream(out)))
+        head = (int(mode), pqk + q_off * 4, lqk, pqk + k_off * 4, lqk, self._ptr(v, torch.float32, "v") + v_off * 4, int(ldv),
+                (pf + gate_off * 4) if gate_off is not None else None, int(ld), (pf + beta_off * 4) if delta else None, int(ld),
+                (pf + dt_off * 4) if delta else None, int(ld), self._ptr(dt_bias, torch.float32, "dt_bias"),
+                self._ptr(a_log, torch.float32, "a_log"), self._ptr(lower, torch.float32, "lower"), self._ptr(norm_w, torch.float32, "norm_w"),
+                self._ptr(out, None, "out"), out.shape[-1], int(out.dtype is torch.float32), self._ptr(state, torch.float32, "state"),
+                self._ptr(row0, torch.int32, "span_row0"), self._ptr(nrows, torch.int32, "span_rows"), int(n),
+                self._ptr(row_seq, torch.int32, "row_seq"), self._ptr(row_pos, torch.int32, "row_pos"))
+        tail = (int(heads), int(qk_heads), int(n_key), int(n_val), float(q_scale), float(eps), self._stream(out))
+        if o_raw is not None:
+            rows = out.shape[0]
+            if o_raw.numel() < rows * heads * n_val:
+                raise RuntimeError("gated_scan: scratch smaller than the step's rows")
+            self.lib.check(self.lib.exl2_gated_scan_cols(*head, int(rows), self._ptr(o_raw, torch.float32, "o_raw"), *tail))
+        else:
+            self.lib.check(self.lib.exl2_gated_scan(*head, *tail))
+
+    def gated_scan_cols_supported(self, n_key: int, n_val: int) -> bool:
+        return bool(self.lib.exl2_gated_scan_cols_supported(int(n_key), int(n_val)))
 
     def graph_begin_capture(self, stream: int | None) -> None:
         self.lib.check(self.lib.exl2_graph_begin_capture(stream))

@@ -392,8 +392,9 @@ class LayeredModel:
         xh = self.buf("xh", (rows, self.width), self.dtype)
         pe = cfg.pair_embedding or {"buckets": 0, "mul_prev": 0, "mul_cur": 0}
         est = cache.norm_state("embed")
+        nb = max(pe["buckets"], 1)                             # (the multipliers reduced first: the hash stays inside 64 bits)
         ext.embed_pair(self.embed, self.pair_table, self.embed_norm, batch.ids, est["prev_token"] if est is not None else None, batch.row_seq,
-                       batch.row_pos, batch.spans_dev, x32, pe["buckets"], pe["mul_prev"], pe["mul_cur"], cfg.embedding_scale,
+                       batch.row_pos, batch.spans_dev, x32, pe["buckets"], pe["mul_prev"] % nb, pe["mul_cur"] % nb, cfg.embedding_scale,
                        cfg.norm_groups, cfg.norm_eps)
         pending = None
         for norm, module, is_mixer, layer in self.sublayers:

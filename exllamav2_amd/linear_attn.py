@@ -24,6 +24,9 @@ from .cache import SlotState
 from .dense_linear import DenseLinear
 
 
+COLS_FROM = 8                                                 # longest span of a step from which the column-split scan is taken
+
+
 class ForgetGateLinearAttention:
     def __init__(self, model, key: str, layer_idx, *, heads: int, dim: int, vdim: int, out_tag: str = "mix.y"):
         self.model, self.ext, self.key, self.layer_idx = model, model.ext, key, layer_idx
@@ -31,6 +34,7 @@ class ForgetGateLinearAttention:
         if heads <= 0 or dim <= 0 or vdim <= 0:
             raise ValueError(f"{key}: {heads} heads of {dim} x {vdim}")
         self.kv_from = None
+        self.cols_ok = self.ext.gated_scan_cols_supported(dim, vdim)
 
     def load(self, get):
         H, dim, vd, width, f32 = self.heads, self.dim, self.vdim, self.model.width, torch.float32
@@ -63,8 +67,10 @@ class ForgetGateLinearAttention:
         n = self.front.out_features
         f = self.front.forward(xh, rows, out=m.buf("mix.f", (rows, n), f32), bias=self.front_bias)             # [zq | zf | v]
         g = m.buf("la.g", (rows, H * vd), m.dtype)
+        # portions of prompts: the walk dealt to (head, value columns) workgroups + a head-norm launch; decoded tokens: one fused launch
+        o_raw = m.buf("la.o", (rows, H * vd), f32) if self.cols_ok and batch.spans_dev[3] >= COLS_FROM else None
         ext.gated_scan(ext.SCAN_FORGET_WRITES, f, n, 0, H * dim, f, n, 2 * H * dim, self.norm_w, g, st["S"], batch.spans_dev,
-                       batch.row_seq, batch.row_pos, H, H, dim, vd, m.norm_eps, lower=self.lower)
+                       batch.row_seq, batch.row_pos, H, H, dim, vd, m.norm_eps, lower=self.lower, o_raw=o_raw)
         return self.o.forward(g, rows, out=m.buf(self.out_tag, (rows, m.width), f32))
 
 
@@ -76,6 +82,7 @@ class GatedDeltaRule:
             raise ValueError(f"{key}: {heads} heads over {kv_heads} query / key heads of {dim} x {vdim}, {taps} taps")
         self.channels = 2 * kv_heads * dim + heads * vdim         # what passes the convolution: [q | k | v]
         self.kv_from = None
+        self.cols_ok = self.ext.gated_scan_cols_supported(dim, vdim)
 
     def load(self, get):
         H, G, dim, vd, width, f32 = self.heads, self.kv_heads, self.dim, self.vdim, self.model.width, torch.float32
@@ -114,7 +121,8 @@ class GatedDeltaRule:
         c = m.buf("la.c", (rows, ch), f32)
         ext.conv_silu_rows(f, n, 0, self.conv_w, None, c, st["tail"], batch.spans_dev, batch.row_seq, batch.row_pos, ch, self.taps)
         g = m.buf("la.g", (rows, H * vd), m.dtype)
+        o_raw = m.buf("la.o", (rows, H * vd), f32) if self.cols_ok and batch.spans_dev[3] >= COLS_FROM else None
         ext.gated_scan(ext.SCAN_DELTA, f, n, 0, G * dim, c, ch, 2 * G * dim, self.norm_w, g, st["S"], batch.spans_dev, batch.row_seq,
                        batch.row_pos, H, G, dim, vd, m.norm_eps, q_scale=dim ** -0.5, gate_off=self.off_g, beta_off=self.off_b,
-                       dt_off=self.off_a, dt_bias=self.dt_bias, a_log=self.a_log, qk=c, ldqk=ch)
+                       dt_off=self.off_a, dt_bias=self.dt_bias, a_log=self.a_log, qk=c, ldqk=ch, o_raw=o_raw)
         return self.o.forward(g, rows, out=m.buf(self.out_tag, (rows, m.width), f32))

@@ -268,3 +268,111 @@ class Oracle:
 
     def drop(self, seq):
         self.seqs.pop(seq, None)
+
+
+# ---- small random models for the tests ---------------------------------------------------------------------------------------
+
+
+def bf16_round(a):
+    u = np.asarray(a, dtype=np.float32).view(np.uint32)
+    return (((u + 0x7fff + ((u >> 16) & 1)) & 0xffff0000).astype(np.uint32)).view(np.float32)
+
+
+def attn_spec(heads=4, kv_heads=2, dim=16, vdim=8, dims=None, base=10000.0, scale=None):
+    return {"dim": dim, "heads": heads, "kv_heads": kv_heads, "rot": {"base": base, "dims": dim if dims is None else dims},
+            "scale": scale if scale is not None else dim ** -0.5, "vdim": vdim}
+
+
+def ssm_spec(heads=4, vdim=8, state=8, groups=2, norm_groups=2, conv=3):
+    return {"conv": conv, "groups": groups, "heads": heads, "norm_groups": norm_groups, "state": state, "vdim": vdim}
+
+
+def parallel_mixer(left=None, right=None, left_scale=1.25, right_scale=0.75):
+    return {"type": "parallel", "mixer": {"left": left or attn_spec(), "left_scale": left_scale, "right": right or ssm_spec(),
+                                          "right_scale": right_scale}}
+
+
+def hgrn2_mixer(heads=3, dim=8, vdim=12):
+    return {"type": "hgrn2", "mixer": {"dim": dim, "heads": heads, "vdim": vdim}}
+
+
+def delta_mixer(heads=4, kv_heads=2, dim=8, vdim=12, conv=3):
+    return {"type": "delta", "mixer": {"conv": conv, "dim": dim, "heads": heads, "kv_heads": kv_heads, "vdim": vdim}}
+
+
+def moe_ff_spec(experts=5, top=2, ff=12, shared=10):
+    ms = {"expert": {"ff": ff}, "kind": "moe", "router": {"experts": experts, "top": top}}
+    if shared:
+        ms["shared"] = {"ff": shared}
+    return ms
+
+
+def layer(mix, ff=None):
+    return dict(mix, mlp=ff)
+
+
+def small_config(layers, width=32, vocab=61, eps=1e-5, groups=2, mult=0.5, taps=3, embed_scale=2.0, buckets=37, mul_prev=31, mul_cur=5):
+    return {"architecture": "Kilurax", "canon": {"taps": taps},
+            "embedding": {"bigram": {"buckets": buckets, "mul_cur": mul_cur, "mul_prev": mul_prev}, "scale": embed_scale},
+            "layers": layers, "norm": {"eps": eps, "groups": groups}, "residual_mult": mult, "vocab": vocab, "width": width}
+
+
+def random_model(cfg: dict, seed: int = 0) -> dict:
+    """name -> float32 array (bfloat16-representable values), shapes from the configuration"""
+    rng = np.random.default_rng(seed)
+    Wd, taps, out = cfg["width"], cfg["canon"]["taps"], {}
+
+    def mat(name, o, i, gain=1.0):
+        out[name] = bf16_round(rng.standard_normal((o, i)) * gain / math.sqrt(i))
+
+    def vec(name, n, centre=0.0, spread=0.1):
+        out[name] = bf16_round(centre + rng.standard_normal(n) * spread)
+
+    def attention(k, m):
+        H, G, dim, vd = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        mat(k + ".q", H * dim, Wd, 2.0); mat(k + ".k", G * dim, Wd, 2.0); mat(k + ".v", G * vd, Wd); mat(k + ".o", Wd, H * vd)
+        vec(k + ".q.b", H * dim, 0.0, 0.3); vec(k + ".k.b", G * dim, 0.0, 0.3); vec(k + ".v.b", G * vd, 0.0, 0.3); vec(k + ".o.b", Wd, 0.0, 0.3)
+
+    def ssm(k, m):
+        H, vd, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
+        inner, ch = H * vd, H * vd + 2 * G * N
+        mat(k + ".in", 2 * inner + 2 * G * N + H, Wd)
+        out[k + ".conv"] = bf16_round(rng.standard_normal((ch, m["conv"])) / math.sqrt(m["conv"]))
+        vec(k + ".conv.b", ch, 0.0, 0.2); vec(k + ".dt_bias", H, -1.0, 0.5); vec(k + ".A_log", H, 0.0, 0.5); vec(k + ".D", H, 1.0, 0.3)
+        vec(k + ".norm", inner, 1.0); mat(k + ".o", Wd, inner)
+
+    out["embed"] = bf16_round(rng.standard_normal((cfg["vocab"], Wd)))
+    out["bigram"] = bf16_round(rng.standard_normal((cfg["embedding"]["bigram"]["buckets"] + 1, Wd)))
+    vec("embed.norm", Wd, 1.0)
+    for i, spec in enumerate(cfg["layers"]):
+        k, m = f"l{i}", spec["mixer"]
+        vec(k + ".norm1", Wd, 1.0); vec(k + ".norm1b", Wd, 1.0)
+        out[k + ".canon1"] = bf16_round(rng.standard_normal((Wd, taps)) * 0.4)
+        if spec["type"] == "parallel":
+            attention(k + ".mix.left", m["left"]); ssm(k + ".mix.right", m["right"])
+        elif spec["type"] == "hgrn2":
+            H, dim, vd = m["heads"], m["dim"], m["vdim"]
+            mat(k + ".mix.q", H * dim, Wd); mat(k + ".mix.f", H * dim, Wd, 2.0); mat(k + ".mix.v", H * vd, Wd)
+            vec(k + ".mix.f.b", H * dim, 1.0, 1.0)
+            out[k + ".mix.lower"] = bf16_round(rng.uniform(0.0, 0.9, size=H * dim))
+            vec(k + ".mix.norm", vd, 1.0); mat(k + ".mix.o", Wd, H * vd)
+        else:
+            H, G, dim, vd = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            mat(k + ".mix.q", G * dim, Wd, 2.0); mat(k + ".mix.k", G * dim, Wd, 2.0); mat(k + ".mix.v", H * vd, Wd, 2.0)
+            for s, n in (("q", G * dim), ("k", G * dim), ("v", H * vd)):
+                out[f"{k}.mix.{s}.conv"] = bf16_round(rng.standard_normal((n, m["conv"])) / math.sqrt(m["conv"]))
+            mat(k + ".mix.b", H, Wd, 2.0); mat(k + ".mix.a", H, Wd); mat(k + ".mix.g", H * vd, Wd, 2.0)
+            vec(k + ".mix.dt_bias", H, -1.0, 0.5); vec(k + ".mix.A_log", H, -1.0, 0.5)
+            vec(k + ".mix.norm", vd, 1.0); mat(k + ".mix.o", Wd, H * vd)
+        ms = spec.get("mlp")
+        if ms is not None:
+            vec(k + ".norm2", Wd, 1.0); vec(k + ".norm2b", Wd, 1.0)
+            out[k + ".canon2"] = bf16_round(rng.standard_normal((Wd, taps)) * 0.4)
+            mat(k + ".mlp.router", ms["router"]["experts"], Wd, 2.0)
+            names = [f"e{e}" for e in range(ms["router"]["experts"])] + (["shared"] if ms.get("shared") else [])
+            for n in names:
+                ff = ms["shared"]["ff"] if n == "shared" else ms["expert"]["ff"]
+                mat(f"{k}.mlp.{n}.gate", ff, Wd, 2.0); mat(f"{k}.mlp.{n}.up", ff, Wd, 2.0); mat(f"{k}.mlp.{n}.down", Wd, ff, 2.0)
+    vec("final.norm", Wd, 1.0)
+    mat("head", cfg["vocab"], Wd)
+    return out
