@@ -206,14 +206,14 @@ KERNEL void __launch_bounds__(256) gated_scan_kernel(const GatedScanArgs a)
 #define GSC_TPW (GSC_CHUNK / 4)              // tokens a wave stages per round
 #define GSC_MAX_N 256                        // key channels: 4 per lane while a wave stages a token, NPT = N / 16 <= 16 rows per thread
 
-template <int NPT, int MODE>
+template <int NPT, int MODE, bool FULL>                      // FULL: N == 16 * NPT, no row of a thread lies outside the state
 KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a, float* o_raw)
 {
     DYN_SMEM(smem);
     const int h = bid_x(), sp = bid_y(), cb = bid_z();
     const int n_tok = a.span_rows[sp], r0 = a.span_row0[sp];
     const int pos0 = a.row_pos[r0];
-    const int P = a.P, N = a.N;
+    const int P = a.P, N = FULL ? GSC_KS * NPT : a.N;
     const int t = tid(), lane = lane_id(), wv = wave_id();
     const int pl = t / GSC_KS, j = t % GSC_KS;
     const int p = cb * GSC_COLS + pl;
@@ -321,6 +321,10 @@ KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a,
         publish();
         block_sync_lds();
         if (c0 + GSC_CHUNK < n_tok) request(c0 + GSC_CHUNK);
+        float* orow = o_raw + (long long)(r0 + c0) * a.heads * P + h * P + p;
+        // (four tokens unrolled: only the state's own update chains from token to token -- the sums that close a read-out and the
+        // LDS reads of the tokens behind overlap with it; two partial sums halve each chain)
+        #pragma unroll 4
         for (int kk = 0; kk < nc; kk++)
         {
             const float vv = s_v[kk * GSC_COLS + pl];
@@ -328,38 +332,44 @@ KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a,
             if (MODE == GS_DELTA)
             {
                 const float g = s_g[kk];
-                float kt = 0.0f;
+                float kt[2] = {0.0f, 0.0f}, o2 = 0.0f;
                 #pragma unroll
                 for (int i = 0; i < NPT; i++)
                 {
                     const int n = j + GSC_KS * i;
-                    if (n < N) { S[i] *= g; kt = fmaf(S[i], s_k[kk * N + n], kt); }
+                    if (FULL || n < N) { S[i] *= g; kt[i & 1] = fmaf(S[i], s_k[kk * N + n], kt[i & 1]); }
                 }
-                kt = row16_allreduce_add(kt);
-                const float u = s_b[kk] * (vv - kt);
+                const float u = s_b[kk] * (vv - row16_allreduce_add(kt[0] + kt[1]));
                 #pragma unroll
                 for (int i = 0; i < NPT; i++)
                 {
                     const int n = j + GSC_KS * i;
-                    if (n < N) { S[i] = fmaf(s_k[kk * N + n], u, S[i]); o = fmaf(S[i], s_q[kk * N + n], o); }
+                    if (FULL || n < N)
+                    {
+                        S[i] = fmaf(s_k[kk * N + n], u, S[i]);
+                        if (i & 1) o2 = fmaf(S[i], s_q[kk * N + n], o2); else o = fmaf(S[i], s_q[kk * N + n], o);
+                    }
                 }
+                o += o2;
             }
             else
             {
+                float o2 = 0.0f;
                 #pragma unroll
                 for (int i = 0; i < NPT; i++)
                 {
                     const int n = j + GSC_KS * i;
-                    if (n < N)
+                    if (FULL || n < N)
                     {
                         const float f = s_k[kk * N + n];
                         S[i] = fmaf(f, S[i], (1.0f - f) * vv);
-                        o = fmaf(S[i], s_q[kk * N + n], o);
+                        if (i & 1) o2 = fmaf(S[i], s_q[kk * N + n], o2); else o = fmaf(S[i], s_q[kk * N + n], o);
                     }
                 }
+                o += o2;
             }
             o = row16_allreduce_add(o);
-            if (owner && j == 0) o_raw[(long long)(r0 + c0 + kk) * a.heads * P + h * P + p] = o;
+            if (owner && j == 0) orow[(long long)kk * a.heads * P] = o;
         }
     }
     #pragma unroll
@@ -489,24 +499,26 @@ extern "C" int exl2_gated_scan_cols(int mode, const float* q, int ldq, const flo
         static bool attr_done[EXL2_MAX_DEVICES];
         if (exl2_first_on_device(attr_done))
         {
-            (void)hipFuncSetAttribute((const void*)gated_scan_cols_kernel<16, GS_FORGET_WRITES>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            (void)hipFuncSetAttribute((const void*)gated_scan_cols_kernel<16, GS_DELTA>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_cols_kernel<16, GS_FORGET_WRITES, false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_cols_kernel<16, GS_DELTA, false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_cols_kernel<16, GS_FORGET_WRITES, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void*)gated_scan_cols_kernel<16, GS_DELTA, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         }
     }
     const dim3 grid(heads, spans, (n_val + GSC_COLS - 1) / GSC_COLS);
     const int npt = (n_key + GSC_KS - 1) / GSC_KS;
+    const bool full = n_key == GSC_KS * 4 || n_key == GSC_KS * 8 || n_key == GSC_KS * 16;
+#define GSC_LAUNCH(NPT_, MODE_) do { if (full) LAUNCH((gated_scan_cols_kernel<NPT_, MODE_, true>), grid, dim3(256), smem, stream, a, o_raw); \
+                                     else LAUNCH((gated_scan_cols_kernel<NPT_, MODE_, false>), grid, dim3(256), smem, stream, a, o_raw); } while (0)
     if (mode == GS_DELTA)
     {
-        if (npt <= 4) LAUNCH((gated_scan_cols_kernel<4, GS_DELTA>), grid, dim3(256), smem, stream, a, o_raw);
-        else if (npt <= 8) LAUNCH((gated_scan_cols_kernel<8, GS_DELTA>), grid, dim3(256), smem, stream, a, o_raw);
-        else LAUNCH((gated_scan_cols_kernel<16, GS_DELTA>), grid, dim3(256), smem, stream, a, o_raw);
+        if (npt <= 4) GSC_LAUNCH(4, GS_DELTA); else if (npt <= 8) GSC_LAUNCH(8, GS_DELTA); else GSC_LAUNCH(16, GS_DELTA);
     }
     else
     {
-        if (npt <= 4) LAUNCH((gated_scan_cols_kernel<4, GS_FORGET_WRITES>), grid, dim3(256), smem, stream, a, o_raw);
-        else if (npt <= 8) LAUNCH((gated_scan_cols_kernel<8, GS_FORGET_WRITES>), grid, dim3(256), smem, stream, a, o_raw);
-        else LAUNCH((gated_scan_cols_kernel<16, GS_FORGET_WRITES>), grid, dim3(256), smem, stream, a, o_raw);
+        if (npt <= 4) GSC_LAUNCH(4, GS_FORGET_WRITES); else if (npt <= 8) GSC_LAUNCH(8, GS_FORGET_WRITES); else GSC_LAUNCH(16, GS_FORGET_WRITES);
     }
+#undef GSC_LAUNCH
     const float* gt = mode == GS_DELTA ? gate : nullptr;
     if (out_f32) LAUNCH(head_norm_gate_kernel<float>, dim3(rows, heads), dim3(64), 0, stream, (const float*)o_raw, norm_w, gt, ldg, out, ldo, heads, n_val, eps);
     else LAUNCH(head_norm_gate_kernel<u16>, dim3(rows, heads), dim3(64), 0, stream, (const float*)o_raw, norm_w, gt, ldg, out, ldo, heads, n_val, eps);

@@ -479,11 +479,24 @@ KERNEL void __launch_bounds__(256) sandwich_norm_vec_kernel(const SandwichArgs a
         if (a.out) wi[e] = ro_ld4<T>((const T*)a.w_in + i);
         if (conv)
         {
-            #pragma unroll
-            for (int k = 0; k < 4; k++)
+            if (a.taps == 4)                                       // a channel's four taps are one 8- or 16-byte load
+            {
                 #pragma unroll
-                for (int j = 0; j < SW_MAX_TAPS; j++)
-                    cw[e][k][j] = j < a.taps ? ro_ld<T>((const T*)a.conv_w + (long long)(i + k) * a.taps + j) : 0.0f;
+                for (int k = 0; k < 4; k++)
+                {
+                    const f32x4 w4 = ro_ld4<T>((const T*)a.conv_w + (long long)(i + k) * 4);
+                    #pragma unroll
+                    for (int j = 0; j < SW_MAX_TAPS; j++) cw[e][k][j] = w4[j];
+                }
+            }
+            else
+            {
+                #pragma unroll
+                for (int k = 0; k < 4; k++)
+                    #pragma unroll
+                    for (int j = 0; j < SW_MAX_TAPS; j++)
+                        cw[e][k][j] = j < a.taps ? ro_ld<T>((const T*)a.conv_w + (long long)(i + k) * a.taps + j) : 0.0f;
+            }
             #pragma unroll
             for (int j = 0; j < SW_MAX_TAPS - 1; j++)
                 tl[e][j] = (j < a.taps - 1 && pos - (a.taps - 1 - j) >= 0) ? *(const f32x4*)(tail + (long long)j * a.width + i) : zero4;
@@ -924,7 +937,7 @@ extern "C" int exl2_sandwich_norm(float* x, const float* y, float ya, const floa
     a.row_pos = row_pos; a.taps = taps; a.width = width; a.groups = groups; a.eps = eps;
     const auto al16 = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
     const bool vec = width % 4 == 0 && width <= 256 * 4 * 4 && (width / groups) % 4 == 0 && groups <= SW_MAX_GROUPS && taps <= SW_MAX_TAPS
-                     && al16(x) && al16(y) && al16(y2) && al16(moe_y) && al16(w_out) && al16(w_in) && al16(out) && al16(tail) && (dtype == 0 || al16(w_in));
+                     && al16(x) && al16(y) && al16(y2) && al16(moe_y) && al16(w_out) && al16(w_in) && al16(out) && al16(tail) && al16(conv_w);
     if (vec)
     {
         const int nc = width <= 1024 ? 1 : width <= 2048 ? 2 : 4;

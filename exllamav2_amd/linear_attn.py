@@ -18,13 +18,16 @@ keeps S -- and the delta rule the last taps - 1 convolution inputs -- in its slo
 constructor parameters."""
 from __future__ import annotations
 
+import os
+
 import torch
 
 from .cache import SlotState
 from .dense_linear import DenseLinear
 
 
-COLS_FROM = 8                                                 # longest span of a step from which the column-split scan is taken
+# longest span of a step from which the column-split scan is taken (EXL2_SCAN_COLS_FROM: kernel-tuning A/B runs)
+COLS_FROM = int(os.environ.get("EXL2_SCAN_COLS_FROM", "1"))
 
 
 class ForgetGateLinearAttention:
@@ -67,7 +70,8 @@ class ForgetGateLinearAttention:
         n = self.front.out_features
         f = self.front.forward(xh, rows, out=m.buf("mix.f", (rows, n), f32), bias=self.front_bias)             # [zq | zf | v]
         g = m.buf("la.g", (rows, H * vd), m.dtype)
-        # portions of prompts: the walk dealt to (head, value columns) workgroups + a head-norm launch; decoded tokens: one fused launch
+        # the walk dealt to (head, value columns) workgroups + a head-norm launch (state shapes outside that kernel, or a raised
+        # COLS_FROM for short spans: the fused launch of one workgroup per head)
         o_raw = m.buf("la.o", (rows, H * vd), f32) if self.cols_ok and batch.spans_dev[3] >= COLS_FROM else None
         ext.gated_scan(ext.SCAN_FORGET_WRITES, f, n, 0, H * dim, f, n, 2 * H * dim, self.norm_w, g, st["S"], batch.spans_dev,
                        batch.row_seq, batch.row_pos, H, H, dim, vd, m.norm_eps, lower=self.lower, o_raw=o_raw)
