@@ -206,7 +206,11 @@ KERNEL void __launch_bounds__(256) gated_scan_kernel(const GatedScanArgs a)
 #define GSC_TPW (GSC_CHUNK / 4)              // tokens a wave stages per round
 #define GSC_MAX_N 256                        // key channels: 4 per lane while a wave stages a token, NPT = N / 16 <= 16 rows per thread
 
-template <int NPT, int MODE, bool FULL>                      // FULL: N == 16 * NPT, no row of a thread lies outside the state
+// rows of the state a thread holds: FULL (N == 16 * NPT, no row outside the state): NPT consecutive ones, so that a token's k and q
+// come as 16-byte LDS reads; otherwise every 16th, guarded
+#define GSC_ROW(i) (FULL ? j * NPT + (i) : j + GSC_KS * (i))
+
+template <int NPT, int MODE, bool FULL>
 KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a, float* o_raw)
 {
     DYN_SMEM(smem);
@@ -230,7 +234,7 @@ KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a,
     #pragma unroll
     for (int i = 0; i < NPT; i++)
     {
-        const int n = j + GSC_KS * i;
+        const int n = GSC_ROW(i);
         S[i] = (owner && pos0 > 0 && n < N) ? st[(long long)n * P + p] : 0.0f;
     }
     const float a_neg = MODE == GS_DELTA ? -expf(a.a_log[h]) : 0.0f, dtb = MODE == GS_DELTA ? a.dt_bias[h] : 0.0f;
@@ -329,26 +333,39 @@ KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a,
         {
             const float vv = s_v[kk * GSC_COLS + pl];
             float o = 0.0f;
+            float kr[NPT], qr[NPT];                              // the token's k (or forget gate) and q at this thread's rows
+            if (FULL)
+            {
+                #pragma unroll
+                for (int c = 0; c < NPT / 4; c++)
+                {
+                    const f32x4 k4 = *(const f32x4*)(s_k + kk * N + j * NPT + 4 * c), q4 = *(const f32x4*)(s_q + kk * N + j * NPT + 4 * c);
+                    #pragma unroll
+                    for (int e = 0; e < 4; e++) { kr[4 * c + e] = k4[e]; qr[4 * c + e] = q4[e]; }
+                }
+            }
+            else
+            {
+                #pragma unroll
+                for (int i = 0; i < NPT; i++)
+                {
+                    const int n = GSC_ROW(i);
+                    kr[i] = n < N ? s_k[kk * N + n] : 0.0f;
+                    qr[i] = n < N ? s_q[kk * N + n] : 0.0f;
+                }
+            }
             if (MODE == GS_DELTA)
             {
                 const float g = s_g[kk];
                 float kt[2] = {0.0f, 0.0f}, o2 = 0.0f;
                 #pragma unroll
-                for (int i = 0; i < NPT; i++)
-                {
-                    const int n = j + GSC_KS * i;
-                    if (FULL || n < N) { S[i] *= g; kt[i & 1] = fmaf(S[i], s_k[kk * N + n], kt[i & 1]); }
-                }
+                for (int i = 0; i < NPT; i++) { S[i] *= g; kt[i & 1] = fmaf(S[i], kr[i], kt[i & 1]); }
                 const float u = s_b[kk] * (vv - row16_allreduce_add(kt[0] + kt[1]));
                 #pragma unroll
                 for (int i = 0; i < NPT; i++)
                 {
-                    const int n = j + GSC_KS * i;
-                    if (FULL || n < N)
-                    {
-                        S[i] = fmaf(s_k[kk * N + n], u, S[i]);
-                        if (i & 1) o2 = fmaf(S[i], s_q[kk * N + n], o2); else o = fmaf(S[i], s_q[kk * N + n], o);
-                    }
+                    S[i] = fmaf(kr[i], u, S[i]);
+                    if (i & 1) o2 = fmaf(S[i], qr[i], o2); else o = fmaf(S[i], qr[i], o);
                 }
                 o += o2;
             }
@@ -358,13 +375,8 @@ KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a,
                 #pragma unroll
                 for (int i = 0; i < NPT; i++)
                 {
-                    const int n = j + GSC_KS * i;
-                    if (FULL || n < N)
-                    {
-                        const float f = s_k[kk * N + n];
-                        S[i] = fmaf(f, S[i], (1.0f - f) * vv);
-                        if (i & 1) o2 = fmaf(S[i], s_q[kk * N + n], o2); else o = fmaf(S[i], s_q[kk * N + n], o);
-                    }
+                    S[i] = fmaf(kr[i], S[i] - vv, vv);           // f S + (1 - f) v (rows outside the state read f = q = 0 and are never stored)
+                    if (i & 1) o2 = fmaf(S[i], qr[i], o2); else o = fmaf(S[i], qr[i], o);
                 }
                 o += o2;
             }
@@ -375,7 +387,7 @@ KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a,
     #pragma unroll
     for (int i = 0; i < NPT; i++)
     {
-        const int n = j + GSC_KS * i;
+        const int n = GSC_ROW(i);
         if (owner && n < N) st[(long long)n * P + p] = S[i];
     }
     (void)pc;

@@ -505,6 +505,44 @@ def test_matrix_core_sizes_in_portions_and_decoding_bf16(be):
     eng.close()
 
 
+def test_head_sizes_of_a_real_model_bf16_and_f32(be):
+    """sizes at which every tuned kernel path is taken (attention tiles of 128, the chunked state-space scan, full-state column scans of
+    64 and 128 key channels, the vector norm, grouped expert launches): a prompt in portions, then decoding, beside a second request"""
+    if be.is_emu:
+        pytest.skip("minutes on the CPU twin; the small configurations cover its logic")
+    cfg = OK.small_config([
+        OK.layer(OK.parallel_mixer(OK.attn_spec(heads=4, kv_heads=2, dim=128, vdim=128, dims=64, base=500000.0),
+                                   OK.ssm_spec(heads=8, vdim=32, state=64, groups=2, norm_groups=2, conv=4)), OK.moe_ff_spec(experts=8, top=2, ff=64, shared=96)),
+        OK.layer(OK.hgrn2_mixer(heads=2, dim=128, vdim=128), OK.moe_ff_spec(experts=8, top=2, ff=64, shared=64)),
+        OK.layer(OK.delta_mixer(heads=4, kv_heads=2, dim=64, vdim=64, conv=4), None),
+        OK.layer(OK.delta_mixer(heads=2, kv_heads=2, dim=128, vdim=128, conv=3), OK.moe_ff_spec(experts=4, top=1, ff=128, shared=None)),
+        OK.layer(OK.hgrn2_mixer(heads=4, dim=64, vdim=64), None)], width=256, vocab=300, groups=2, taps=4, buckets=251, mul_prev=127, mul_cur=7)
+    W = OK.random_model(cfg, seed=61)
+    reqs = {"a": clear_tokens(cfg, W, 150, 62, gap=0.002), "b": clear_tokens(cfg, W, 20, 63, gap=0.002)}
+    oracle = OK.Oracle(cfg, W)
+    want = {r: oracle.feed(r, t) for r, t in reqs.items()}
+    for dtype in (F32, BF16):
+        eng = make_engine(be, cfg, W, dtype, max_tokens=512, page=64, graphs=True)
+        got = {r: {} for r in reqs}
+
+        def step(parts, end=()):
+            lg = be.n(eng.step([(r, reqs[r][lo:hi], list(range(hi - lo))) for r, lo, hi in parts], end))
+            k = 0
+            for r, lo, hi in parts:
+                for p in range(lo, hi):
+                    got[r][p] = lg[k]; k += 1
+
+        step([("a", 0, 70)])
+        step([("a", 70, 135), ("b", 0, 9)])
+        step([("a", 135, 137), ("b", 9, 10)])
+        for i in range(10):
+            step([("a", 137 + i, 138 + i), ("b", 10 + i, 11 + i)])
+        step([("a", 147, 150)])
+        for r in reqs:
+            assert ok(np.stack([got[r][p] for p in range(len(reqs[r]))]), want[r], dtype), (r, dtype)
+        eng.close()
+
+
 def crafted_model(seed=31):
     """one layer of attention beside a (silenced) state-space scan, made so that token 0's query matches token 1's key and nothing
     else: queries read inputs 0-3, keys inputs 4-7 through the same matrix, values the other inputs; token 0 is marked in inputs 0-3,
