@@ -419,8 +419,8 @@ def sandwich_config(s: dict) -> dict:
         else:
             layers.append({"type": "delta", "mixer": {"conv": 4, "dim": s["la_dim"], "heads": s["la_heads"], "kv_heads": s["la_kv_heads"],
                                                       "vdim": s["la_vdim"]}, "mlp": ff})
-    return {"architecture": "Kilurax", "canon": {"taps": 4}, "embedding": {"bigram": {"buckets": 65521, "mul_cur": 7, "mul_prev": 127}, "scale": 1.0},
-            "layers": layers, "norm": {"eps": 1e-6, "groups": 2}, "residual_mult": 0.5, "vocab": s["vocab"], "width": s["width"]}
+    return {"architecture": "Kilurax", "canon": {"taps": 4}, "embedding": {"bigram": {"buckets": 65521, "mul_cur": 11, "mul_prev": 131}, "scale": 1.0},
+            "layers": layers, "norm": {"eps": 1e-5, "groups": 2}, "residual_mult": 0.7, "vocab": s["vocab"], "width": s["width"]}
 
 
 def sandwich_random_tensors(cfg: dict, device, seed: int = 0) -> dict:

@@ -274,18 +274,28 @@ KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a,
 
     auto publish = [&]()
     {
+        // (the sums of squares of all the wave's tokens first, then their reductions side by side: sixteen independent exchanges
+        // instead of a chain of them)
+        float sq[GSC_TPW], sk[GSC_TPW];
+        if (MODE == GS_DELTA)
+        {
+            #pragma unroll
+            for (int u = 0; u < GSC_TPW; u++)
+            {
+                sq[u] = sk[u] = 0.0f;
+                #pragma unroll
+                for (int e = 0; e < GSC_MAX_N / 64; e++) { sq[u] = fmaf(rq[u][e], rq[u][e], sq[u]); sk[u] = fmaf(rk[u][e], rk[u][e], sk[u]); }
+            }
+            #pragma unroll
+            for (int u = 0; u < GSC_TPW; u++) { sq[u] = wave_allreduce_add(sq[u]); sk[u] = wave_allreduce_add(sk[u]); }
+        }
         #pragma unroll
         for (int u = 0; u < GSC_TPW; u++)
         {
             const int kk = wv + 4 * u;
             if (MODE == GS_DELTA)
             {
-                float sq = 0.0f, sk = 0.0f;
-                #pragma unroll
-                for (int e = 0; e < GSC_MAX_N / 64; e++) { sq = fmaf(rq[u][e], rq[u][e], sq); sk = fmaf(rk[u][e], rk[u][e], sk); }
-                sq = wave_allreduce_add(sq);
-                sk = wave_allreduce_add(sk);
-                const float mq = a.q_scale / sqrtf(sq + 1e-6f), mk = 1.0f / sqrtf(sk + 1e-6f);
+                const float mq = a.q_scale / sqrtf(sq[u] + 1e-6f), mk = 1.0f / sqrtf(sk[u] + 1e-6f);
                 #pragma unroll
                 for (int e = 0; e < GSC_MAX_N / 64; e++)
                 {

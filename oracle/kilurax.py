@@ -311,7 +311,7 @@ def layer(mix, ff=None):
     return dict(mix, mlp=ff)
 
 
-def small_config(layers, width=32, vocab=61, eps=1e-5, groups=2, mult=0.5, taps=3, embed_scale=2.0, buckets=37, mul_prev=31, mul_cur=5):
+def small_config(layers, width=32, vocab=61, eps=1e-5, groups=2, mult=0.625, taps=3, embed_scale=2.0, buckets=37, mul_prev=31, mul_cur=5):
     return {"architecture": "Kilurax", "canon": {"taps": taps},
             "embedding": {"bigram": {"buckets": buckets, "mul_cur": mul_cur, "mul_prev": mul_prev}, "scale": embed_scale},
             "layers": layers, "norm": {"eps": eps, "groups": groups}, "residual_mult": mult, "vocab": vocab, "width": width}
