@@ -25,7 +25,7 @@ template <> DEV void gs_st<float>(float* p, float v) { *p = v; }
 DEV float gs_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
 DEV float gs_softplus(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
 
-#define GS_CHUNK 16                          // tokens staged in LDS per round
+#define GS_CHUNK 16                          // tokens staged in LDS at a time
 #define GS_MAX_NPT 256                       // state rows per thread
 #define GS_MAX_N 1024                        // key channels per head (16 per lane while a wave normalises a token's q and k)
 
@@ -196,14 +196,14 @@ KERNEL void __launch_bounds__(256) gated_scan_kernel(const GatedScanArgs a)
 // The value columns of a head's state never meet inside the recurrence (u_p = beta (v_p - S[:, p] . k), o_p = S[:, p] . q), so a
 // span's walk is dealt to (head, block of GSC_COLS columns) workgroups: GSC_KS = 16 lanes share a column, each holds N / 16 rows in
 // registers, and a token costs a thread a handful of fused multiply-adds and four lane exchanges per sum instead of a pass over
-// N / 2 rows.  Tokens are taken GSC_CHUNK at a time; the raw projections of the NEXT round are requested into registers before a round
+// N / 2 rows.  Tokens are taken GSC_CHUNK at a time; the raw projections of the NEXT batch of tokens are requested into registers before a batch
 // is stepped through, so their latency hides behind it, and turned into gates / unit vectors / decays when they are written to LDS.
 // The raw read-out goes to o_raw fp32 [rows, heads * P]; the head norm needs the whole head and is head_norm_gate_kernel's.
 
 #define GSC_KS 16
 #define GSC_COLS 16                          // 256 threads = 16 columns x 16 lanes
 #define GSC_CHUNK 32
-#define GSC_TPW (GSC_CHUNK / 4)              // tokens a wave stages per round
+#define GSC_TPW (GSC_CHUNK / 4)              // tokens a wave stages at a time
 #define GSC_MAX_N 256                        // key channels: 4 per lane while a wave stages a token, NPT = N / 16 <= 16 rows per thread
 
 // rows of the state a thread holds: FULL (N == 16 * NPT, no row outside the state): NPT consecutive ones, so that a token's k and q
@@ -238,7 +238,7 @@ KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a,
         S[i] = (owner && pos0 > 0 && n < N) ? st[(long long)n * P + p] : 0.0f;
     }
     const float a_neg = MODE == GS_DELTA ? -expf(a.a_log[h]) : 0.0f, dtb = MODE == GS_DELTA ? a.dt_bias[h] : 0.0f;
-    // what a thread keeps of the next round while the current one is stepped through
+    // what a thread keeps of the next batch of tokens while the current one is stepped through
     float rq[GSC_TPW][GSC_MAX_N / 64], rk[GSC_TPW][GSC_MAX_N / 64], rv[2], rb = 0.0f, rd = 0.0f;
     const int qh = MODE == GS_DELTA ? hq : h;
 
@@ -331,7 +331,7 @@ KERNEL void __launch_bounds__(256) gated_scan_cols_kernel(const GatedScanArgs a,
     for (int c0 = 0; c0 < n_tok; c0 += GSC_CHUNK)
     {
         const int nc = min(GSC_CHUNK, n_tok - c0);
-        block_sync_lds();                                        // the round before has been stepped through by every thread
+        block_sync_lds();                                        // the batch before has been stepped through by every thread
         publish();
         block_sync_lds();
         if (c0 + GSC_CHUNK < n_tok) request(c0 + GSC_CHUNK);
@@ -493,7 +493,7 @@ extern "C" int exl2_gated_scan_cols_supported(int n_key, int n_val)
     return n_key > 0 && n_key <= GSC_MAX_N && n_val > 0 ? 1 : 0;
 }
 
-/* exl2_gated_scan for portions of prompts: a span's walk dealt to (head, 16 value columns) workgroups, the next round's inputs in
+/* exl2_gated_scan for portions of prompts: a span's walk dealt to (head, 16 value columns) workgroups, the next tokens' inputs in
    flight behind the current one; the head norm (and gate) as a second launch over o_raw (scratch, fp32 [rows, heads * n_val]).  Same
    operands and results as exl2_gated_scan (sums associate differently: results agree to rounding). */
 extern "C" int exl2_gated_scan_cols(int mode, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* gate,

@@ -626,7 +626,7 @@ int exl2_gated_scan(int mode, const float* q, int ldq, const float* k, int ldk, 
                     const int* span_row0, const int* span_rows, int spans, const int* row_seq, const int* row_pos, int heads,
                     int qk_heads, int n_key, int n_val, float q_scale, float eps, void* stream);
 /* exl2_gated_scan for portions of prompts: a span's walk is dealt to (head, 16 value columns) workgroups (the columns of the state
-   never meet inside the recurrence), 16 lanes share a column, the next round's inputs are in flight behind the current one; the head
+   never meet inside the recurrence), 16 lanes share a column, the next tokens' inputs are in flight behind the current ones; the head
    norm (and gate) runs as a second launch over o_raw (scratch, fp32 [rows, heads * n_val]).  State shapes for which
    exl2_gated_scan_cols_supported returns 1; results agree with exl2_gated_scan to rounding. */
 int exl2_gated_scan_cols_supported(int n_key, int n_val);
